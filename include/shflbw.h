@@ -1,0 +1,210 @@
+/*
+ * shflbw.h -- C ABI of the MI355X (gfx950) Shfl-BW sparse inference library.
+ *
+ * Shfl-BW weights: an M x K fp16 matrix stored as row panels of `brow` (V) rows;
+ * inside a panel only some V x 1 column vectors are kept; an optional row
+ * permutation says which logical output row each stored row is.  Two
+ * operators: SpMM  D = A_sparse * B_dense (+ C)  and SpConv2D (implicit GEMM).
+ *
+ * Every entry point below replaces one piece of the host API of the reference
+ * library (hgyhungry/ShflBW_Sparse_NN, paths relative to its root); the
+ * citation says which.  Plain pointers and sizes only; all functions return a
+ * shflbw_status (0 = success) and never terminate the process.
+ *
+ * fp16 data crosses this boundary as raw IEEE binary16 bit patterns
+ * (uint16_t on the host, 2-byte elements on the device).
+ */
+#ifndef SHFLBW_H
+#define SHFLBW_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum shflbw_status {
+    SHFLBW_OK = 0,
+    SHFLBW_ERR_INVALID = 1,     /* null pointer / bad argument */
+    SHFLBW_ERR_SHAPE = 2,       /* shape precondition violated (nrow % brow, N % 8, ...) */
+    SHFLBW_ERR_STATE = 3,       /* object not initialised / not synced to the device */
+    SHFLBW_ERR_HIP = 4,         /* a HIP runtime call failed; see shflbw_last_error() */
+    SHFLBW_ERR_UNSUPPORTED = 5, /* block size / layout without a kernel */
+    SHFLBW_ERR_FORMAT = 6,      /* malformed text dump or inconsistent arrays */
+    SHFLBW_ERR_CAPACITY = 7     /* caller buffer too small */
+} shflbw_status;
+
+/* Human readable text for a status; and the detail of the last failure on this thread. */
+const char* shflbw_status_string(int status);
+const char* shflbw_last_error(void);
+
+/* ------------------------------------------------------------------------- *
+ * Mask generator.  Replaces block_sparse/util/random_mask.h:4-10
+ * (random_mask, 12- and 9-argument forms; util/random_mask.cc:10-67).
+ * indptr: X+1 ints (X = nrow/brow); indices: `indices_cap` ints.
+ * ------------------------------------------------------------------------- */
+int shflbw_random_mask_ex(int nrow, int ncol, int brow, int bcol, float block_density,
+                          int block_divisor, int block_padding, unsigned seed,
+                          int* nnzb, int* padded_nnzb, int* indptr, int* indices, size_t indices_cap);
+int shflbw_random_mask(int nrow, int ncol, int brow, int bcol, float block_density, unsigned seed,
+                       int* nnzb, int* indptr, int* indices, size_t indices_cap);
+
+/* ------------------------------------------------------------------------- *
+ * Weight container.  Replaces BlockwiseSpMatrix<half>
+ * (block_sparse/spmm/blockwise_format.h:13-68) and BlockwiseSpFilter<half>
+ * (block_sparse/spconv/blockwise_format.h:17-27).  The object owns its host
+ * arrays and its device buffers; shflbw_weight_destroy frees both
+ * (blockwise_format.h:48-58).
+ * ------------------------------------------------------------------------- */
+typedef struct shflbw_weight shflbw_weight;
+
+typedef struct shflbw_weight_info {
+    int nrow, ncol, nnzb, brow, bcol;
+    float density;
+    unsigned seed;
+    int row_permute;
+    int initialized, device_synced;
+    int F, R, S, C; /* filter view (nrow = F, ncol = R*S*C); all 0 for a plain matrix */
+} shflbw_weight_info;
+
+/* Device pointers of a synced weight: DeviceRef, blockwise_format.h:35-42. */
+typedef struct shflbw_device_ref {
+    void* meta;                 /* indptr | indices*bcol | row_permute_ids, 8-int aligned sections */
+    void* data;                 /* values, verbatim */
+    const int* csb_indptr;      /* X+1 */
+    const int* csb_indices;     /* nnzb, pre-multiplied by bcol */
+    const int* row_permute_ids; /* nrow, or NULL when not permuted */
+    const void* csb_values;     /* nnzb*brow*bcol fp16 */
+} shflbw_device_ref;
+
+int shflbw_weight_create(shflbw_weight** out);
+void shflbw_weight_destroy(shflbw_weight* w);
+
+/* BlockwiseSpMatrix::init_random, blockwise_format.h:70-123: mask, permutation
+ * (iota + std::shuffle with default_random_engine(seed)), values rand()%9-4. */
+int shflbw_weight_init_random(shflbw_weight* w, int nrow, int ncol, int brow, int bcol,
+                              float expected_density, int row_permute, unsigned seed);
+/* BlockwiseSpFilter::init_random, spconv/blockwise_format.h:30-52 (matrix is F x (R*S*C),
+ * column k = (r*S + s)*C + c). */
+int shflbw_filter_init_random(shflbw_weight* w, int F, int R, int S, int C, int brow, int bcol,
+                              float expected_density, int filter_permute, unsigned seed);
+/* Build from caller arrays (what `load` does from text).  values: nnzb*brow*bcol fp16 bit
+ * patterns, column-major inside each block (blockwise_format.h:297).  row_permute_ids may be
+ * NULL (not permuted).  For a filter pass R,S,C (> 0) with ncol == R*S*C; else 0,0,0. */
+int shflbw_weight_set(shflbw_weight* w, int nrow, int ncol, int brow, int bcol, int nnzb,
+                      const int* indptr, const int* indices, const uint16_t* values,
+                      const int* row_permute_ids, int R, int S, int C);
+/* Replace the values only (same pattern); drops a previous device image. */
+int shflbw_weight_set_values(shflbw_weight* w, const uint16_t* values, size_t count);
+
+/* BlockwiseSpMatrix::dump / load, blockwise_format.h:125-198 (text format of
+ * example/spmatrix_dump_load.md).  dump: writes at most `cap` bytes (no terminator) and
+ * always reports the size needed. */
+int shflbw_weight_dump_text(const shflbw_weight* w, char* buf, size_t cap, size_t* needed);
+int shflbw_weight_load_text(shflbw_weight* w, const char* text, size_t len);
+
+int shflbw_weight_get_info(const shflbw_weight* w, shflbw_weight_info* info);
+/* Borrowed pointers to the host arrays (valid until the weight is re-initialised/destroyed). */
+int shflbw_weight_host_arrays(const shflbw_weight* w, const int** indptr, const int** indices,
+                              const uint16_t** values, const int** row_permute_ids);
+/* config_str, blockwise_format.h:105-114 / spconv/blockwise_format.h:42-51. */
+const char* shflbw_weight_config_str(const shflbw_weight* w);
+
+/* transform_and_sync_device, blockwise_format.h:200-266: packs the meta image, uploads
+ * meta + values, and additionally builds the private MFMA-ordered image the gfx950 kernels
+ * read.  meta_host: the packed host image (meta_h), valid after a sync. */
+int shflbw_weight_sync_device(shflbw_weight* w);
+int shflbw_weight_meta_host(const shflbw_weight* w, const int** meta, size_t* n_ints);
+int shflbw_weight_device_ref(const shflbw_weight* w, shflbw_device_ref* ref);
+
+/* ------------------------------------------------------------------------- *
+ * SpMM.  Replaces SpmmBlockwiseOpState (spmm/blockwise_op.h:6-17),
+ * SpmmBlockwiseOp::initialize / operator() (:81-174) and
+ * SpmmBlockwiseInitFn / SpmmBlockwiseExecFn (:188-215).
+ *   D[row_permute_ids[r]][:] = alpha * (A_stored[r,:] * B) + beta * C[row_permute_ids[r]][:]
+ * B: K x N row-major fp16, C/D: M x N row-major fp16, all device pointers, caller owned.
+ * Preconditions: weight synced; bcol == 1; N % 8 == 0; B, C, D 16-byte aligned.
+ * The state is a copyable POD holding raw pointers; it dangles if the weight is
+ * re-initialised or destroyed (same as the reference).
+ * ------------------------------------------------------------------------- */
+typedef struct shflbw_spmm_state {
+    size_t shared_mem_size;
+    unsigned grid_dim[3];
+    unsigned block_dim[3];
+    int init_success;
+    int variant; /* native tile variant chosen for this problem */
+    struct {
+        int M, N, K;
+        const void* A_values;
+        const void* B;
+        const void* C;
+        void* D;
+        const int* A_bsr_indptr;
+        const int* A_bsr_indices;
+        const int* A_row_indices;
+        float alpha, beta;
+    } args;
+    /* private device image (owned by the weight) */
+    const void* packed_values;
+    const int* packed_indices;
+    const int* panel_ptr;
+    int brow;
+} shflbw_spmm_state;
+
+/* C may be NULL when beta == 0.  variant < 0 selects automatically. */
+int shflbw_spmm_init(shflbw_spmm_state* state, const shflbw_weight* w, int N,
+                     const void* B, const void* C, void* D, float alpha, float beta);
+int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, int N,
+                             const void* B, const void* C, void* D, float alpha, float beta, int variant);
+/* Asynchronous launch on `stream` (a hipStream_t, NULL = default stream); launch only:
+ * no allocation, no synchronisation (benchmark loop, benchmark/benchmark.spmm.cu:29-42). */
+int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream);
+/* Number of native tile variants available for a block size, and a short name for each. */
+int shflbw_spmm_variant_count(int brow);
+const char* shflbw_spmm_variant_name(int brow, int variant);
+
+/* ------------------------------------------------------------------------- *
+ * SpConv2D as implicit GEMM.  Replaces SpconvBlockwiseOpState
+ * (spconv/blockwise_op.h:6-17), SpconvBlockwiseOp::initialize / operator() (:79-149)
+ * and SpconvBlockwiseInitFn / ExecFn (:161-193).
+ *   GEMM view: M = F, K = R*S*C ordered (r, s, c), N = B*Ho*Wo; alpha = 1, beta = 0.
+ *   Tensors are NHWC: IFMap[b][hi][wi][c], OFMap[b][ho][wo][f] (fp16, device, caller owned).
+ *   H, W are the INPUT extents; padding is R/2, S/2 ("same" for stride 1, as the
+ *   reference's col2im, spconv/conv_format.h:77-81); Ho = (H + 2*(R/2) - R)/stride + 1.
+ * Preconditions: filter synced, bcol == 1, C % 8 == 0, F % 8 == 0.
+ * ------------------------------------------------------------------------- */
+typedef struct shflbw_spconv_state {
+    size_t shared_mem_size;
+    unsigned grid_dim[3];
+    unsigned block_dim[3];
+    int init_success;
+    int variant;
+    struct {
+        int B, H, W, C, F, R, S, stride;
+        const void* A_values;
+        const void* IFMap;
+        void* OFMap;
+        const int* A_bsr_indptr;
+        const int* A_bsr_indices;
+        const int* A_row_indices;
+        float alpha, beta;
+    } args;
+    int Ho, Wo;
+    const void* packed_values;
+    const int* packed_indices;
+    const int* panel_ptr;
+    int brow;
+} shflbw_spconv_state;
+
+int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* filter,
+                       int B, int H, int W, int stride, const void* IFMap, void* OFMap);
+int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream);
+
+/* Library / device facts (for logs): compute units, clock (kHz), LDS bytes per workgroup. */
+int shflbw_device_info(int* compute_units, int* clock_khz, size_t* lds_bytes, char* arch, size_t arch_cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHFLBW_H */

@@ -1,0 +1,359 @@
+// Device side of the C ABI: uploads of the weight images and the SpMM / SpConv
+// init + exec entry points.  Reference: block_sparse/spmm/blockwise_format.h:230-266
+// (upload), block_sparse/spmm/blockwise_op.h:81-215 and
+// block_sparse/spconv/blockwise_op.h:79-193 (init / exec).
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "shflbw.h"
+#include "spconv_launch.h"
+#include "spmm_launch.h"
+#include "weight_internal.h"
+
+namespace shflbw {
+
+#define SHFLBW_HIP_TRY(expr)                                                                            \
+    do {                                                                                                \
+        hipError_t e_ = (expr);                                                                         \
+        if (e_ != hipSuccess) {                                                                         \
+            set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__);       \
+            return SHFLBW_ERR_HIP;                                                                      \
+        }                                                                                               \
+    } while (0)
+
+void clear_device(shflbw_weight* w)
+{
+    void** bufs[] = {&w->d_meta, &w->d_values, &w->d_group_ptr, &w->d_packed_indices, &w->d_packed_values};
+    for (void** b : bufs) {
+        if (*b) (void)hipFree(*b);
+        *b = nullptr;
+    }
+}
+
+static int upload_one(void** dst, const void* src, size_t bytes)
+{
+    // zero-length arrays (an empty matrix) still get a valid pointer
+    SHFLBW_HIP_TRY(hipMalloc(dst, bytes ? bytes : 16));
+    if (bytes) SHFLBW_HIP_TRY(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+    return SHFLBW_OK;
+}
+
+int upload(shflbw_weight* w)
+{
+    int rc;
+    if ((rc = upload_one(&w->d_meta, w->meta_h.data(), w->meta_h.size() * sizeof(int))) ||
+        (rc = upload_one(&w->d_values, w->values.data(), w->values.size() * sizeof(uint16_t))) ||
+        (rc = upload_one(&w->d_group_ptr, w->group_ptr.data(), w->group_ptr.size() * sizeof(int))) ||
+        (rc = upload_one(&w->d_packed_indices, w->packed_indices.data(), w->packed_indices.size() * sizeof(int))) ||
+        (rc = upload_one(&w->d_packed_values, w->packed_values.data(), w->packed_values.size() * sizeof(uint16_t)))) {
+        clear_device(w);
+        return rc;
+    }
+    return SHFLBW_OK;
+}
+
+static const SpmmVariant* find_spmm_variant(int brow, int variant, int* n_for_brow)
+{
+    int count = 0;
+    const SpmmVariant* all = spmm_variants(&count);
+    const SpmmVariant* hit = nullptr;
+    int seen = 0;
+    for (int i = 0; i < count; i++) {
+        if (all[i].V != brow) continue;
+        if (seen == variant) hit = &all[i];
+        seen++;
+    }
+    if (n_for_brow) *n_for_brow = seen;
+    return hit;
+}
+
+static const SpconvVariant* find_spconv_variant(int brow, int variant, int* n_for_brow)
+{
+    int count = 0;
+    const SpconvVariant* all = spconv_variants(&count);
+    const SpconvVariant* hit = nullptr;
+    int seen = 0;
+    for (int i = 0; i < count; i++) {
+        if (all[i].V != brow) continue;
+        if (seen == variant) hit = &all[i];
+        seen++;
+    }
+    if (n_for_brow) *n_for_brow = seen;
+    return hit;
+}
+
+// Tile choice when the caller does not force one: the widest column tile that still
+// gives every compute unit work, falling back to narrower tiles for small N.
+static int auto_spmm_variant(int brow, int X, int N)
+{
+    int n = 0;
+    find_spmm_variant(brow, 0, &n);
+    for (int v = 0; v < n; v++) {
+        const SpmmVariant* s = find_spmm_variant(brow, v, nullptr);
+        const long wgs = (long)X * ((N + s->BN - 1) / s->BN);
+        if (wgs >= 256 || v == n - 1) return v;
+    }
+    return 0;
+}
+
+} // namespace shflbw
+
+using namespace shflbw;
+
+extern "C" {
+
+int shflbw_spmm_variant_count(int brow)
+{
+    int n = 0;
+    find_spmm_variant(brow, 0, &n);
+    return n;
+}
+
+const char* shflbw_spmm_variant_name(int brow, int variant)
+{
+    const SpmmVariant* v = find_spmm_variant(brow, variant, nullptr);
+    return v ? v->name : "";
+}
+
+int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C,
+                             void* D, float alpha, float beta, int variant)
+{
+    if (!state) return SHFLBW_ERR_INVALID;
+    memset(state, 0, sizeof(*state));
+    if (!w || !B || !D) {
+        set_error("spmm_init: null weight, B or D");
+        return SHFLBW_ERR_INVALID;
+    }
+    if (!w->device_synced) { // assert at blockwise_op.h:87
+        set_error("spmm_init: sparse matrix is not synced to device");
+        return SHFLBW_ERR_STATE;
+    }
+    if (w->bcol != 1) { // assert at blockwise_op.h:86 (BK = 1)
+        set_error("spmm_init: bcol must be 1 (got %d)", w->bcol);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (N <= 0 || (N % 8) != 0) {
+        set_error("spmm_init: N must be a positive multiple of 8 (got %d)", N);
+        return SHFLBW_ERR_SHAPE;
+    }
+    if (beta != 0.f && !C) {
+        set_error("spmm_init: beta != 0 needs C");
+        return SHFLBW_ERR_INVALID;
+    }
+    if (((uintptr_t)B | (uintptr_t)D | (uintptr_t)C) & 15) {
+        set_error("spmm_init: B, C and D must be 16-byte aligned");
+        return SHFLBW_ERR_INVALID;
+    }
+    const int X = w->nrow / w->brow;
+    if (variant < 0) variant = auto_spmm_variant(w->brow, X, N);
+    const SpmmVariant* v = find_spmm_variant(w->brow, variant, nullptr);
+    if (!v) {
+        set_error("spmm_init: no tile variant %d for block size %d", variant, w->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    SHFLBW_HIP_TRY(v->prepare());
+
+    shflbw_device_ref ref;
+    shflbw_weight_device_ref(w, &ref);
+    state->args.M = w->nrow;
+    state->args.N = N;
+    state->args.K = w->ncol;
+    state->args.A_values = ref.csb_values;
+    state->args.B = B;
+    state->args.C = C;
+    state->args.D = D;
+    state->args.A_bsr_indptr = ref.csb_indptr;
+    state->args.A_bsr_indices = ref.csb_indices;
+    state->args.A_row_indices = ref.row_permute_ids;
+    state->args.alpha = alpha;
+    state->args.beta = beta;
+    state->packed_values = w->d_packed_values;
+    state->packed_indices = (const int*)w->d_packed_indices;
+    state->panel_ptr = (const int*)w->d_group_ptr;
+    state->brow = w->brow;
+    state->variant = variant;
+    state->shared_mem_size = (size_t)v->lds_bytes;
+    state->grid_dim[0] = (unsigned)(X * ((N + v->BN - 1) / v->BN));
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[0] = (unsigned)v->threads;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
+int shflbw_spmm_init(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C, void* D,
+                     float alpha, float beta)
+{
+    return shflbw_spmm_init_variant(state, w, N, B, C, D, alpha, beta, -1);
+}
+
+int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
+{
+    if (!state || !state->init_success) {
+        set_error("spmm_exec: state was not initialised successfully");
+        return SHFLBW_ERR_STATE;
+    }
+    const SpmmVariant* v = find_spmm_variant(state->brow, state->variant, nullptr);
+    if (!v) return SHFLBW_ERR_UNSUPPORTED;
+    SpmmLaunchArgs a;
+    a.M = state->args.M;
+    a.N = state->args.N;
+    a.K = state->args.K;
+    a.X = a.M / state->brow;
+    a.n_tiles = 0;
+    a.packedA = (const half8_t*)state->packed_values;
+    a.kidx = state->packed_indices;
+    a.group_ptr = state->panel_ptr;
+    a.indptr = state->args.A_bsr_indptr;
+    a.row_ids = state->args.A_row_indices;
+    a.B = (const half_t*)state->args.B;
+    a.C = (const half_t*)state->args.C;
+    a.D = (half_t*)state->args.D;
+    a.alpha = state->args.alpha;
+    a.beta = state->args.beta;
+    if (a.X == 0) return SHFLBW_OK;
+    hipError_t e = v->launch(a, (hipStream_t)stream);
+    if (e != hipSuccess) {
+        set_error("spmm_exec: launch failed: %s", hipGetErrorString(e));
+        return SHFLBW_ERR_HIP;
+    }
+    return SHFLBW_OK;
+}
+
+int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                       const void* IFMap, void* OFMap)
+{
+    if (!state) return SHFLBW_ERR_INVALID;
+    memset(state, 0, sizeof(*state));
+    if (!f || !IFMap || !OFMap) {
+        set_error("spconv_init: null filter, IFMap or OFMap");
+        return SHFLBW_ERR_INVALID;
+    }
+    if (!f->device_synced) { // assert at spconv/blockwise_op.h:83
+        set_error("spconv_init: sparse filter is not synced to device");
+        return SHFLBW_ERR_STATE;
+    }
+    if (f->R <= 0) {
+        set_error("spconv_init: weight has no filter view (use shflbw_filter_init_random or pass R,S,C to shflbw_weight_set)");
+        return SHFLBW_ERR_STATE;
+    }
+    if (f->bcol != 1) {
+        set_error("spconv_init: bcol must be 1 (got %d)", f->bcol);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (B <= 0 || H <= 0 || W <= 0 || stride <= 0) {
+        set_error("spconv_init: non-positive B, H, W or stride");
+        return SHFLBW_ERR_INVALID;
+    }
+    if ((f->C % 8) != 0 || (f->F % 8) != 0) {
+        set_error("spconv_init: C and F must be multiples of 8 (got %d, %d)", f->C, f->F);
+        return SHFLBW_ERR_SHAPE;
+    }
+    if (((uintptr_t)IFMap | (uintptr_t)OFMap) & 15) {
+        set_error("spconv_init: IFMap and OFMap must be 16-byte aligned");
+        return SHFLBW_ERR_INVALID;
+    }
+    const int Ho = (H + 2 * (f->R / 2) - f->R) / stride + 1;
+    const int Wo = (W + 2 * (f->S / 2) - f->S) / stride + 1;
+    if (Ho <= 0 || Wo <= 0) {
+        set_error("spconv_init: empty output (%d x %d)", Ho, Wo);
+        return SHFLBW_ERR_SHAPE;
+    }
+    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
+    if (!v) {
+        set_error("spconv_init: no kernel for block size %d", f->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    SHFLBW_HIP_TRY(v->prepare());
+    shflbw_device_ref ref;
+    shflbw_weight_device_ref(f, &ref);
+    state->args.B = B;
+    state->args.H = H;
+    state->args.W = W;
+    state->args.C = f->C;
+    state->args.F = f->F;
+    state->args.R = f->R;
+    state->args.S = f->S;
+    state->args.stride = stride;
+    state->args.A_values = ref.csb_values;
+    state->args.IFMap = IFMap;
+    state->args.OFMap = OFMap;
+    state->args.A_bsr_indptr = ref.csb_indptr;
+    state->args.A_bsr_indices = ref.csb_indices;
+    state->args.A_row_indices = ref.row_permute_ids;
+    state->args.alpha = 1.f; // spconv/blockwise_op.h:89-94
+    state->args.beta = 0.f;
+    state->Ho = Ho;
+    state->Wo = Wo;
+    state->packed_values = f->d_packed_values;
+    state->packed_indices = (const int*)f->d_packed_indices;
+    state->panel_ptr = (const int*)f->d_group_ptr;
+    state->brow = f->brow;
+    state->variant = 0;
+    state->shared_mem_size = (size_t)v->lds_bytes;
+    const long npix = (long)B * Ho * Wo;
+    state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[0] = (unsigned)v->threads;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
+int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
+{
+    if (!state || !state->init_success) {
+        set_error("spconv_exec: state was not initialised successfully");
+        return SHFLBW_ERR_STATE;
+    }
+    const SpconvVariant* v = find_spconv_variant(state->brow, state->variant, nullptr);
+    if (!v) return SHFLBW_ERR_UNSUPPORTED;
+    SpconvLaunchArgs a;
+    a.B = state->args.B;
+    a.H = state->args.H;
+    a.W = state->args.W;
+    a.C = state->args.C;
+    a.F = state->args.F;
+    a.R = state->args.R;
+    a.S = state->args.S;
+    a.stride = state->args.stride;
+    a.pad_h = a.R / 2;
+    a.pad_w = a.S / 2;
+    a.Ho = state->Ho;
+    a.Wo = state->Wo;
+    a.X = a.F / state->brow;
+    a.n_tiles = 0;
+    a.packedA = (const half8_t*)state->packed_values;
+    a.kidx = state->packed_indices;
+    a.group_ptr = state->panel_ptr;
+    a.indptr = state->args.A_bsr_indptr;
+    a.row_ids = state->args.A_row_indices;
+    a.in = (const half_t*)state->args.IFMap;
+    a.out = (half_t*)state->args.OFMap;
+    hipError_t e = v->launch(a, (hipStream_t)stream);
+    if (e != hipSuccess) {
+        set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));
+        return SHFLBW_ERR_HIP;
+    }
+    return SHFLBW_OK;
+}
+
+int shflbw_device_info(int* compute_units, int* clock_khz, size_t* lds_bytes, char* arch, size_t arch_cap)
+{
+    int dev = 0;
+    SHFLBW_HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t p;
+    SHFLBW_HIP_TRY(hipGetDeviceProperties(&p, dev));
+    if (compute_units) *compute_units = p.multiProcessorCount;
+    if (clock_khz) *clock_khz = p.clockRate;
+    if (lds_bytes) *lds_bytes = p.sharedMemPerBlock;
+    if (arch && arch_cap) {
+        strncpy(arch, p.gcnArchName, arch_cap - 1);
+        arch[arch_cap - 1] = 0;
+    }
+    return SHFLBW_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,72 @@
+// Device-side building blocks shared by the gfx950 SpMM and SpConv kernels.
+// Wave = 64 lanes.  Matrix cores are driven as D' = Bfrag x Afrag (activation rows,
+// weight columns), so one lane ends up holding consecutive output columns of one
+// output row, which makes the fp16 conversion and the LDS-staged row scatter cheap.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace shflbw {
+
+typedef _Float16 half_t;
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+#define SHFLBW_LDS __attribute__((address_space(3)))
+// read-only data addressed uniformly by a wave: loads through this address space are scalar
+#define SHFLBW_CONST __attribute__((address_space(4)))
+
+// s_waitcnt immediate that waits only for the vector-memory counter to drop to n
+// (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
+__device__ __forceinline__ constexpr int vmcnt_imm(int n)
+{
+    return (n & 0xf) | (0x7 << 4) | (0xf << 8) | ((n >> 4) << 14);
+}
+
+// XOR mask, in 32-byte units, applied to the position of a piece inside its LDS row.
+// Rows r, r+1, r+2, r+3 (r % 4 == 0) read by one transposing load then touch eight
+// distinct 32-byte bank groups for the two neighbouring column halves, both when the
+// LDS serves 128 B and when it serves 256 B per clock.
+__device__ __forceinline__ constexpr int row_xor32(int row_mod4)
+{
+    return 2 * row_mod4 + (row_mod4 >> 1); // 0, 2, 5, 7
+}
+
+// Transposing LDS load: inside each group of 16 lanes, lane i supplies the address of
+// four consecutive halves of row i/4 (piece i%4 of a 4 x 16 block) and receives column
+// i of that block (rows 0..3).
+__device__ __forceinline__ half4_t lds_read_tr16(uint32_t byte_addr)
+{
+    short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SHFLBW_LDS short4_t*)(uintptr_t)byte_addr);
+    return __builtin_bit_cast(half4_t, v);
+}
+
+// One wave instruction moves 64 x 16 bytes from per-lane global addresses to 1 KiB of
+// consecutive LDS starting at the wave-uniform byte address `lds_base` (lane l lands at
+// +16 l).  Issued as inline assembly on purpose: the compiler then neither counts it nor
+// orders LDS reads after it, so the kernels place exact `s_waitcnt vmcnt(n)` themselves
+// and keep several stages in flight.  M0 carries the LDS address; one wait state is
+// required between the scalar write of M0 and the load.  No "memory" clobber: the
+// statement is ordered against barriers and explicit waits because it is volatile, and
+// a clobber would stop the compiler from using scalar loads for read-only metadata.
+__device__ __forceinline__ void global_to_lds_16B(const void* gptr, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_base)
+                 : "m0");
+}
+
+// Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs; this makes consecutive *logical* ids share an XCD (and
+// therefore its L2), so tiles that gather the same activation slab run side by side.
+__device__ __forceinline__ int xcd_local_id(int wg, int total)
+{
+    const int per = total >> 3;
+    return (wg < (per << 3)) ? (wg & 7) * per + (wg >> 3) : wg;
+}
+
+} // namespace shflbw

@@ -1,0 +1,278 @@
+// Shfl-BW SpMM for gfx950 (MI355X):  D[perm[r]] = alpha * (A_stored[r,:] * B) + beta * C[perm[r]].
+//
+// Replaces the reference's kernel and its device primitives
+// (block_sparse/spmm/blockwise_kernel.h:108-294 main loop, :552-579 epilogue,
+// block_sparse/common/{mma,memcpy,swizzle,epilogue}.h) with a design for 64-lane waves:
+//
+//  * one workgroup = one row panel (V stored rows) x BN output columns; its waves split BN;
+//  * the kept activation rows B[k, n0:n0+BN] are gathered straight from global memory into a
+//    ring of LDS stages (16 bytes per lane, no register round trip), KT rows per stage;
+//  * a wave reads its B operand with transposing LDS loads (the rows are n-contiguous, the
+//    matrix core wants 8 consecutive k per lane), the 32-byte pieces of each LDS row are
+//    XOR-swizzled so these loads are bank-conflict free;
+//  * the A operand comes from the weight's private image, already in register order: each
+//    fragment is 1 KiB that one wave instruction copies into the stage next to the B rows;
+//  * the kept-column ids are wave-uniform per gathered row and come through scalar loads, so
+//    the vector-memory counter only ever counts the LDS copies and the waits are exact;
+//  * fp32 accumulators are rounded once to fp16, staged through LDS and scattered as whole
+//    row segments through the permutation.
+#include "kernel_common.h"
+#include "spmm_launch.h"
+
+namespace shflbw {
+
+template <int V, int WN, int NWAVES, int KT, int NSTAGE>
+struct SpmmCfg {
+    static constexpr int BN = WN * NWAVES;
+    static constexpr int MB = V / 32;        // 32-row blocks of the panel
+    static constexpr int NB = WN / 32;       // 32-column blocks of a wave's slice
+    static constexpr int ROWB = BN * 2;      // bytes of one gathered row in LDS
+    static constexpr int CPR = BN / 8;       // 16-byte pieces per row
+    static constexpr int RPI = 64 / CPR > 0 ? 64 / CPR : 1; // rows covered by one gather instruction
+    static constexpr int IPR = CPR / 64 > 0 ? CPR / 64 : 1; // gather instructions per row (BN > 512)
+    static constexpr int SPT = KT / 16;         // MFMA k-steps per stage
+    static constexpr int B_BYTES = KT * ROWB;   // gathered rows of one stage
+    static constexpr int A_FRAGS = SPT * MB;    // 1 KiB A fragments of one stage
+    static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
+    static constexpr int INSTR = KT * CPR / 64; // 1 KiB gather instructions per stage
+    static constexpr int IPW = INSTR / NWAVES;  // ... issued by each wave
+    static constexpr int RPW = KT / NWAVES;     // gathered rows owned by each wave
+    static constexpr int AIPW = (A_FRAGS + NWAVES - 1) / NWAVES; // A fragment copies per wave
+    static constexpr int DMA_PER_ITER = IPW + AIPW;              // per wave and stage
+    static constexpr int EPI_ROWB = ROWB + 16;  // padded row of the output staging tile
+    static constexpr int PIPE_BYTES = NSTAGE * STAGE_BYTES;
+    static constexpr int EPI_BYTES = V * EPI_ROWB;
+    static constexpr int LDS_BYTES = PIPE_BYTES > EPI_BYTES ? PIPE_BYTES : EPI_BYTES;
+    static constexpr int THREADS = NWAVES * 64;
+    static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
+    static_assert(BN >= 128 && BN <= 512 && (BN & (BN - 1)) == 0, "row swizzle needs 8..32 32-byte pieces per row");
+    static_assert(KT % 16 == 0 && 64 % KT == 0, "stage depth must divide the 64-slot padding");
+    static_assert(KT % NWAVES == 0 && INSTR % NWAVES == 0, "gather must split evenly over the waves");
+    static_assert(IPW * RPI == RPW, "a wave's gather instructions cover whole rows");
+    static_assert((NSTAGE - 2) * DMA_PER_ITER < 64, "vmcnt is a 6-bit counter");
+    static_assert(NSTAGE >= 2, "double buffering at least");
+};
+
+template <int V, int WN, int NWAVES, int KT, int NSTAGE>
+__global__ void __launch_bounds__(NWAVES * 64) spmm_shflbw_kernel(SpmmLaunchArgs a)
+{
+    using Cfg = SpmmCfg<V, WN, NWAVES, KT, NSTAGE>;
+    constexpr int BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, ROWB = Cfg::ROWB, CPR = Cfg::CPR;
+    constexpr int IPW = Cfg::IPW, SPT = Cfg::SPT, EPI_ROWB = Cfg::EPI_ROWB, RPI = Cfg::RPI, RPW = Cfg::RPW;
+    constexpr int AIPW = Cfg::AIPW, A_FRAGS = Cfg::A_FRAGS;
+
+    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lid = xcd_local_id(blockIdx.x, a.X * a.n_tiles);
+    const int nt = lid / a.X;
+    const int panel = lid - nt * a.X;
+    const int n0 = nt * BN;
+    const int N = a.N;
+
+    const int nnz = a.indptr[panel + 1] - a.indptr[panel];
+    const int g0 = a.group_ptr[panel];
+    const SHFLBW_CONST int* kidx =
+        (const SHFLBW_CONST int*)(uintptr_t)(a.kidx + (size_t)g0 * 64 + wave * RPW); // this wave's rows of a stage
+    const char* __restrict__ pA = (const char*)a.packedA + (size_t)g0 * (64 * V * 2) + lane * 16;
+    const int nsteps = (nnz + 15) >> 4;
+    const int ntiles = (nsteps + SPT - 1) / SPT;
+
+    // ---- per-lane constants of the gather.  Instruction j of this wave fills LDS pieces
+    // (wave*IPW + j)*64 + lane of the stage; `sub` says which of the RPI rows the lane is in.
+    const int sub = lane / CPR;
+    int gcol[IPW];
+#pragma unroll
+    for (int j = 0; j < IPW; j++) {
+        const int piece = ((wave * IPW + j) << 6) + lane;
+        const int row = piece / CPR, pc = piece % CPR;
+        const int lc = ((((pc >> 1) ^ row_xor32(row & 3))) << 1) | (pc & 1);
+        const int col = n0 + lc * 8;
+        gcol[j] = col < N ? col : 0; // columns past N are never stored; keep the address valid
+    }
+    // ---- per-lane constants of the transposing loads
+    const int li = lane & 15;
+    uint32_t boff[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        const int unit = (wave * WN + nb * 32) / 16 + ((lane >> 4) & 1);
+        boff[nb] = (uint32_t)((8 * (lane >> 5) + (li >> 2)) * ROWB + ((unit ^ row_xor32(li >> 2)) << 5) + ((li & 3) << 3));
+    }
+
+    float16_t acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.f;
+
+    // kept-column ids of this wave's rows for the tile that is gathered next (scalar loads)
+    int ks[RPW];
+    auto load_idx = [&](int tile) {
+#pragma unroll
+        for (int r = 0; r < RPW; r++) ks[r] = kidx[tile * KT + r];
+    };
+    // all copies of one stage issued by this wave: its rows of B and its share of the A fragments
+    auto fill_stage = [&](int tile, int stage) {
+        const uint32_t sb = lds0 + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < AIPW; j++) {
+            const int f = (wave * AIPW + j) % A_FRAGS; // surplus waves repeat a fragment (same bytes)
+            global_to_lds_16B(pA + ((size_t)tile * A_FRAGS + f) * 1024, sb + Cfg::B_BYTES + f * 1024);
+        }
+#pragma unroll
+        for (int j = 0; j < IPW; j++) {
+            int k = ks[j * RPI];
+#pragma unroll
+            for (int q = 1; q < RPI; q++) k = (sub == q) ? ks[j * RPI + q] : k;
+            global_to_lds_16B(a.B + ((size_t)k * N + gcol[j]), sb + (wave * IPW + j) * 1024);
+        }
+    };
+
+    // ---- prologue: fill NSTAGE-1 stages
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; s++) {
+        if (s < ntiles) {
+            load_idx(s);
+            fill_stage(s, s);
+        }
+    }
+    if (NSTAGE - 1 < ntiles) load_idx(NSTAGE - 1);
+
+    int stage = 0;         // stage holding tile t
+    int fill = NSTAGE - 1; // stage that receives tile t + NSTAGE - 1
+    for (int t = 0; t < ntiles; t++) {
+        // this wave's copies of tile t must have landed; the (NSTAGE-2) stages issued after it
+        // may stay in flight (they did get issued if tile t+NSTAGE-2 exists)
+        if (t + NSTAGE - 2 < ntiles)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * Cfg::DMA_PER_ITER));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads(); // every wave's share of tile t is in LDS; stage `fill` is no longer read
+
+        if (t + NSTAGE - 1 < ntiles) {
+            fill_stage(t + NSTAGE - 1, fill);
+            if (t + NSTAGE < ntiles) load_idx(t + NSTAGE);
+        }
+
+        const uint32_t sb = lds0 + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < SPT; kk++) {
+            if (t * SPT + kk < nsteps) {
+                half8_t afrag[MB], bfrag[NB];
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+                    afrag[mb] = *(SHFLBW_LDS half8_t*)(uintptr_t)(sb + Cfg::B_BYTES + (kk * MB + mb) * 1024 + lane * 16);
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) {
+                    const half4_t lo = lds_read_tr16(sb + boff[nb] + (kk * 16) * ROWB);
+                    const half4_t hi = lds_read_tr16(sb + boff[nb] + (kk * 16 + 4) * ROWB);
+                    bfrag[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag[nb], afrag[mb], acc[mb][nb], 0, 0, 0);
+            }
+        }
+        stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
+        fill = (fill + 1 == NSTAGE) ? 0 : fill + 1;
+    }
+
+    // ---- epilogue: fp32 -> fp16 once, stage the V x BN tile in LDS, scatter row segments
+    __syncthreads(); // all waves are done reading the pipeline stages
+    const float alpha = a.alpha;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int ig = 0; ig < 4; ig++) {
+                half4_t h;
+#pragma unroll
+                for (int e = 0; e < 4; e++) h[e] = (half_t)(acc[mb][nb][ig * 4 + e] * alpha);
+                const int m = mb * 32 + (lane & 31);
+                const int n = wave * WN + nb * 32 + ig * 8 + (lane >> 5) * 4;
+                *(SHFLBW_LDS half4_t*)(uintptr_t)(lds0 + m * EPI_ROWB + n * 2) = h;
+            }
+    __syncthreads();
+    const float beta = a.beta;
+    constexpr int PIECES = V * CPR;
+#pragma unroll 4
+    for (int id = threadIdx.x; id < PIECES; id += Cfg::THREADS) {
+        const int r = id / CPR, pc = id % CPR;
+        const int col = n0 + pc * 8;
+        if (col < N) {
+            half8_t v = *(SHFLBW_LDS half8_t*)(uintptr_t)(lds0 + r * EPI_ROWB + pc * 16);
+            const int srow = panel * V + r;
+            const int orow = a.row_ids ? a.row_ids[srow] : srow;
+            const size_t off = (size_t)orow * N + col;
+            if (beta != 0.f) {
+                const half8_t c = *(const half8_t*)(a.C + off);
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = (half_t)((float)v[e] + beta * (float)c[e]);
+            }
+            *(half8_t*)(a.D + off) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// variant table
+// ---------------------------------------------------------------------------------------
+template <int V, int WN, int NWAVES, int KT, int NSTAGE>
+static hipError_t launch_variant(const SpmmLaunchArgs& a, hipStream_t stream)
+{
+    using Cfg = SpmmCfg<V, WN, NWAVES, KT, NSTAGE>;
+    const int n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    SpmmLaunchArgs b = a;
+    b.n_tiles = n_tiles;
+    hipLaunchKernelGGL((spmm_shflbw_kernel<V, WN, NWAVES, KT, NSTAGE>), dim3(a.X * n_tiles), dim3(Cfg::THREADS),
+                       Cfg::LDS_BYTES, stream, b);
+    return hipGetLastError();
+}
+
+template <int V, int WN, int NWAVES, int KT, int NSTAGE>
+static hipError_t prepare_variant()
+{
+    using Cfg = SpmmCfg<V, WN, NWAVES, KT, NSTAGE>;
+    return hipFuncSetAttribute((const void*)spmm_shflbw_kernel<V, WN, NWAVES, KT, NSTAGE>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+}
+
+#define SHFLBW_VARIANT(V, WN, NW, KT, NS)                                                                   \
+    {                                                                                                       \
+        V, WN* NW, NW * 64, SpmmCfg<V, WN, NW, KT, NS>::LDS_BYTES, #V "x" #WN "x" #NW "w_k" #KT "_s" #NS,       \
+            &launch_variant<V, WN, NW, KT, NS>, &prepare_variant<V, WN, NW, KT, NS>                          \
+    }
+
+static const SpmmVariant g_variants[] = {
+    // block 64
+    SHFLBW_VARIANT(64, 64, 4, 32, 3),
+    SHFLBW_VARIANT(64, 64, 4, 32, 2),
+    SHFLBW_VARIANT(64, 64, 4, 16, 4),
+    SHFLBW_VARIANT(64, 128, 2, 32, 3),
+    SHFLBW_VARIANT(64, 128, 4, 16, 3),
+    SHFLBW_VARIANT(64, 64, 2, 32, 3),
+    SHFLBW_VARIANT(64, 32, 4, 32, 3),
+    // block 32
+    SHFLBW_VARIANT(32, 64, 4, 32, 3),
+    SHFLBW_VARIANT(32, 128, 2, 32, 3),
+    SHFLBW_VARIANT(32, 128, 4, 16, 3),
+    SHFLBW_VARIANT(32, 64, 2, 32, 3),
+    // block 128
+    SHFLBW_VARIANT(128, 64, 4, 32, 3),
+    SHFLBW_VARIANT(128, 32, 4, 32, 3),
+};
+
+const SpmmVariant* spmm_variants(int* count)
+{
+    *count = (int)(sizeof(g_variants) / sizeof(g_variants[0]));
+    return g_variants;
+}
+
+} // namespace shflbw

@@ -1,0 +1,35 @@
+// Launch-side description of the native SpMM tile variants (host + device shared).
+#pragma once
+#include <hip/hip_runtime.h>
+#include "kernel_common.h"
+
+namespace shflbw {
+
+struct SpmmLaunchArgs {
+    int M, N, K;
+    int X;       // row panels = M / V
+    int n_tiles; // column tiles, filled by the launcher
+    const half8_t* packedA; // private image: A fragments in register order
+    const int* kidx;        // private image: kept column ids, 64-slot padded per panel
+    const int* group_ptr;   // X+1, cumulative 64-slot groups
+    const int* indptr;      // X+1, reference-format panel offsets (for the true nnz)
+    const int* row_ids;     // M, or null when rows are not permuted
+    const half_t* B;
+    const half_t* C;
+    half_t* D;
+    float alpha, beta;
+};
+
+struct SpmmVariant {
+    int V;           // block size (rows per panel)
+    int BN;          // output columns per workgroup
+    int threads;     // workgroup size
+    int lds_bytes;   // dynamic LDS
+    const char* name;
+    hipError_t (*launch)(const SpmmLaunchArgs&, hipStream_t);
+    hipError_t (*prepare)(); // raises the dynamic-LDS limit of the kernel
+};
+
+const SpmmVariant* spmm_variants(int* count);
+
+} // namespace shflbw

@@ -1,0 +1,58 @@
+// Internal definition of the weight container behind the C ABI (shflbw_weight).
+// Host side of the Shfl-BW format: reference block_sparse/spmm/blockwise_format.h:13-68.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "shflbw.h"
+
+struct shflbw_weight {
+    // shape and pattern (blockwise_format.h:15-22)
+    int nrow = 0, ncol = 0, nnzb = 0, brow = 0, bcol = 0;
+    float density = 0.f;
+    unsigned seed = 0;
+    bool row_permute = false;
+    int F = 0, R = 0, S = 0, C = 0; // filter view, spconv/blockwise_format.h:19-23
+
+    // original format on host (:25-27)
+    std::vector<int> indptr, indices, row_permute_ids;
+    std::vector<uint16_t> values; // fp16 bits, column-major inside each block
+
+    // reference-format image (:29-31): indptr | indices*bcol | row_permute_ids
+    std::vector<int> meta_h;
+
+    // private image for the gfx950 kernels, built by sync_device
+    std::vector<int> group_ptr;      // X+1: cumulative count of 64-slot groups per panel
+    std::vector<int> packed_indices; // 64 * group_ptr[X]; tail slots repeat the panel's last id
+    std::vector<uint16_t> packed_values; // 64 * brow * group_ptr[X]; MFMA fragment order, tail zero
+
+    bool initialized = false, device_synced = false;
+    std::string config_str;
+
+    // device buffers (owned)
+    void* d_meta = nullptr;
+    void* d_values = nullptr;
+    void* d_group_ptr = nullptr;
+    void* d_packed_indices = nullptr;
+    void* d_packed_values = nullptr;
+};
+
+namespace shflbw {
+
+void set_error(const char* fmt, ...);
+
+// fp16 bit helpers (IEEE binary16, round to nearest even)
+float half_to_float(uint16_t h);
+uint16_t float_to_half(float f);
+
+// k-extent of one MFMA step for a block size: 32x32x16 tiles for V >= 32, 16x16x32 for V == 16
+inline int mfma_kstep(int brow) { return brow >= 32 ? 16 : 32; }
+
+// builds group_ptr / packed_indices / packed_values from the host arrays
+int build_packed_image(shflbw_weight* w);
+
+// frees device buffers (blockwise_format.h:48-52)
+void clear_device(shflbw_weight* w);
+
+} // namespace shflbw

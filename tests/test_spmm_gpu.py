@@ -1,0 +1,123 @@
+"""GPU parity of the HIP SpMM against the CPU oracle, through the C ABI.
+
+Integer-valued inputs (the reference's own test distribution, test/test.spmm.blockwise.cu and
+cuda_array.h:62-66) must match the oracle bit for bit after one fp16 rounding: this is the
+check of index, padding and permutation handling.  Float inputs are held to the stated
+tolerances.
+"""
+import numpy as np
+import pytest
+
+import shflbw_sparse_nn_amd as S
+from oracle import oracle as O
+from tests import problems as P
+from tests.gpu_util import float_error_report, run_spmm
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2        # max relative error on elements that are not near-cancelled (north star)
+SCALED_TOL = 2.0 ** -9  # |err| / sum|a b|: one fp16 rounding (2^-11) plus fp32 summation order
+
+
+def _exact_case(torch, M, N, K, V, d, permute, variant=-1, seed=2021):
+    w = P.make_weight(M, K, V, d, permute, seed, integer=True)
+    B = P.make_dense(K, N, seed, integer=True)
+    ref = O.float_to_half(P.spmm_oracle(w, B))
+    got = run_spmm(torch, w, B, variant=variant)
+    assert not np.isnan(got.astype(np.float32)).any(), "kernel left output elements unwritten"
+    np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+# the reference's own test case: N = 960 exercises the column-residue path
+@pytest.mark.parametrize("V", [32, 64, 128])
+@pytest.mark.parametrize("permute", [False, True])
+def test_reference_case_all_variants(torch_gpu, V, permute):
+    for variant in range(len(S.spmm_variants(V))):
+        print("variant", variant, S.spmm_variants(V)[variant], flush=True)
+        _exact_case(torch_gpu, 1024, 960, 1024, V, 0.1, permute, variant)
+
+
+@pytest.mark.parametrize("M,N,K,V,d", [
+    (64, 8, 16, 64, 1.0),       # one panel, one partial k-step, tiny N
+    (128, 264, 96, 32, 0.5),    # N residue of 8
+    (256, 512, 200, 64, 0.03),  # panels with very few (possibly zero) vectors
+    (256, 128, 1024, 128, 0.3),
+    (512, 1032, 777, 32, 0.2),  # K not a multiple of anything
+    (1024, 1024, 1024, 64, 0.25),  # cfg0 shape
+])
+def test_exact_shapes(torch_gpu, M, N, K, V, d):
+    _exact_case(torch_gpu, M, N, K, V, d, True)
+
+
+def test_dense_density_is_permuted_gemm(torch_gpu):
+    # d = 1.0: a plain dense GEMM with permuted output rows
+    M, N, K, V = 128, 256, 128, 64
+    w = P.make_weight(M, K, V, 1.0, True, 7, integer=True)
+    B = P.make_dense(K, N, 7, integer=True)
+    got = run_spmm(torch_gpu, w, B).astype(np.float32)
+    A = O.densify(w)
+    np.testing.assert_array_equal(got, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+
+
+def test_empty_panels_write_zeros(torch_gpu):
+    M, N, K, V = 256, 128, 64, 64
+    X = M // V
+    indptr = np.array([0, 0, 3, 3, 3], dtype=np.int32)  # only panel 1 keeps vectors
+    indices = np.array([1, 5, 63], dtype=np.int32)
+    rng = np.random.default_rng(3)
+    w = dict(nrow=M, ncol=K, brow=V, bcol=1, nnzb=3, indptr=indptr, indices=indices,
+             values=rng.integers(-4, 5, size=3 * V).astype(np.float16), row_permute_ids=O.row_permutation(M, 5))
+    B = P.make_dense(K, N, 3, integer=True)
+    got = run_spmm(torch_gpu, w, B)
+    ref = O.float_to_half(P.spmm_oracle(w, B))
+    np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16))
+    assert X == 4 and (got[np.sort(w["row_permute_ids"][:V])] == 0).all()
+
+
+@pytest.mark.parametrize("permute", [False, True])
+def test_beta_c_epilogue(torch_gpu, permute):
+    # D = A*B + C, the overload the reference's example uses (example/spmm.blockwise.cu:50)
+    M, N, K, V = 256, 256, 256, 32
+    w = P.make_weight(M, K, V, 0.2, permute, 11, integer=True)
+    B = P.make_dense(K, N, 11, integer=True)
+    Cm = P.make_dense(M, N, 11, integer=True, stream=3)
+    got = run_spmm(torch_gpu, w, B, Cmat=Cm)
+    ref = O.float_to_half(P.spmm_oracle(w, B, Cm, 1.0, 1.0))
+    np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16))
+    got2 = run_spmm(torch_gpu, w, B, Cmat=Cm, alpha=2.0, beta=-0.5)
+    ref2 = O.float_to_half(P.spmm_oracle(w, B, Cm, 2.0, -0.5))
+    np.testing.assert_array_equal(got2.view(np.uint16), ref2.view(np.uint16))
+
+
+@pytest.mark.parametrize("name", ["cfg0", "cfg1", "cfg2"])
+def test_graded_configs(torch_gpu, name):
+    c = P.SPMM_CONFIGS[name]
+    # integer twin: bit exact
+    _exact_case(torch_gpu, c["M"], c["N"], c["K"], c["V"], c["d"], True)
+    # float inputs as specified
+    w = P.make_weight(c["M"], c["K"], c["V"], c["d"], True, 2021, dist=c["a_dist"])
+    B = P.make_dense(c["K"], c["N"], 2021, dist=c["b_dist"])
+    ref = P.spmm_oracle(w, B)
+    got = run_spmm(torch_gpu, w, B)
+    rel, scaled = float_error_report(got, ref, P.abs_products_bound(w, B))
+    print(name, "max rel err (|ref| >= 1e-2 rms):", rel, " max err / sum|ab|:", scaled, flush=True)
+    assert rel <= REL_TOL
+    assert scaled <= SCALED_TOL
+
+
+def test_linearity_full_size(torch_gpu):
+    # size-independent property at the headline size: A*(B1 + B2) == A*B1 + A*B2, exactly.
+    # B1 and B2 have disjoint supports and entries in {-1, 0, 1}, A has integers in [-4, 4]:
+    # every sum stays below 2048 in magnitude, so all three results are exact in fp16.
+    c = P.SPMM_CONFIGS["cfg1"]
+    w = P.make_weight(c["M"], c["K"], c["V"], c["d"], True, 2021, integer=True)
+    assert 4 * int(np.max(np.diff(w["indptr"]))) < 2048
+    rng = np.random.default_rng(99)
+    X = rng.integers(-1, 2, size=(c["K"], c["N"]))
+    sel = rng.integers(0, 2, size=(c["K"], c["N"]))
+    B1 = (X * sel).astype(np.float16)
+    B2 = (X * (1 - sel)).astype(np.float16)
+    d1 = run_spmm(torch_gpu, w, B1).astype(np.float32)
+    d2 = run_spmm(torch_gpu, w, B2).astype(np.float32)
+    d12 = run_spmm(torch_gpu, w, (B1 + B2).astype(np.float16)).astype(np.float32)
+    np.testing.assert_array_equal(d12, d1 + d2)
