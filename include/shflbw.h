@@ -148,6 +148,7 @@ typedef struct shflbw_spmm_state {
     /* private device image (owned by the weight) */
     const void* packed_values;
     const int* packed_indices;
+    const int* packed_indices_pm;
     const int* panel_ptr;
     int brow;
 } shflbw_spmm_state;

@@ -51,8 +51,8 @@ class _SpmmArgs(C.Structure):
 class SpmmState(C.Structure):
     _fields_ = [("shared_mem_size", C.c_size_t), ("grid_dim", C.c_uint * 3), ("block_dim", C.c_uint * 3),
                 ("init_success", C.c_int), ("variant", C.c_int), ("args", _SpmmArgs),
-                ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("panel_ptr", C.c_void_p),
-                ("brow", C.c_int)]
+                ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("packed_indices_pm", C.c_void_p),
+                ("panel_ptr", C.c_void_p), ("brow", C.c_int)]
 
 
 class _SpconvArgs(C.Structure):

@@ -25,7 +25,8 @@ namespace shflbw {
 
 void clear_device(shflbw_weight* w)
 {
-    void** bufs[] = {&w->d_meta, &w->d_values, &w->d_group_ptr, &w->d_packed_indices, &w->d_packed_values};
+    void** bufs[] = {&w->d_meta, &w->d_values, &w->d_group_ptr, &w->d_packed_indices, &w->d_packed_indices_pm,
+                     &w->d_packed_values};
     for (void** b : bufs) {
         if (*b) (void)hipFree(*b);
         *b = nullptr;
@@ -45,13 +46,30 @@ int upload(shflbw_weight* w)
     int rc;
     if ((rc = upload_one(&w->d_meta, w->meta_h.data(), w->meta_h.size() * sizeof(int))) ||
         (rc = upload_one(&w->d_values, w->values.data(), w->values.size() * sizeof(uint16_t))) ||
-        (rc = upload_one(&w->d_group_ptr, w->group_ptr.data(), w->group_ptr.size() * sizeof(int))) ||
+        (rc = upload_one(&w->d_group_ptr, w->panel_desc.data(), w->panel_desc.size() * sizeof(int))) ||
         (rc = upload_one(&w->d_packed_indices, w->packed_indices.data(), w->packed_indices.size() * sizeof(int))) ||
+        (rc = upload_one(&w->d_packed_indices_pm, w->packed_indices_pm.data(),
+                         w->packed_indices_pm.size() * sizeof(int))) ||
         (rc = upload_one(&w->d_packed_values, w->packed_values.data(), w->packed_values.size() * sizeof(uint16_t)))) {
         clear_device(w);
         return rc;
     }
     return SHFLBW_OK;
+}
+
+// compute units of the current device, looked up once per process
+static int device_compute_units()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cached = n;
+        else
+            cached = 256;
+    }
+    return cached;
 }
 
 static const SpmmVariant* find_spmm_variant(int brow, int variant, int* n_for_brow)
@@ -84,17 +102,13 @@ static const SpconvVariant* find_spconv_variant(int brow, int variant, int* n_fo
     return hit;
 }
 
-// Tile choice when the caller does not force one: the widest column tile that still
-// gives every compute unit work, falling back to narrower tiles for small N.
+// Tile choice when the caller does not force one: the table lists the preferred
+// (persistent, widest) variant of every block size first.
 static int auto_spmm_variant(int brow, int X, int N)
 {
-    int n = 0;
-    find_spmm_variant(brow, 0, &n);
-    for (int v = 0; v < n; v++) {
-        const SpmmVariant* s = find_spmm_variant(brow, v, nullptr);
-        const long wgs = (long)X * ((N + s->BN - 1) / s->BN);
-        if (wgs >= 256 || v == n - 1) return v;
-    }
+    (void)brow;
+    (void)X;
+    (void)N;
     return 0;
 }
 
@@ -171,6 +185,7 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     state->args.beta = beta;
     state->packed_values = w->d_packed_values;
     state->packed_indices = (const int*)w->d_packed_indices;
+    state->packed_indices_pm = (const int*)w->d_packed_indices_pm;
     state->panel_ptr = (const int*)w->d_group_ptr;
     state->brow = w->brow;
     state->variant = variant;
@@ -205,14 +220,15 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
     a.n_tiles = 0;
     a.packedA = (const half8_t*)state->packed_values;
     a.kidx = state->packed_indices;
-    a.group_ptr = state->panel_ptr;
-    a.indptr = state->args.A_bsr_indptr;
+    a.kidx_pm = state->packed_indices_pm;
+    a.panel_desc = state->panel_ptr;
     a.row_ids = state->args.A_row_indices;
     a.B = (const half_t*)state->args.B;
     a.C = (const half_t*)state->args.C;
     a.D = (half_t*)state->args.D;
     a.alpha = state->args.alpha;
     a.beta = state->args.beta;
+    a.num_cus = device_compute_units();
     if (a.X == 0) return SHFLBW_OK;
     hipError_t e = v->launch(a, (hipStream_t)stream);
     if (e != hipSuccess) {
@@ -327,8 +343,7 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.n_tiles = 0;
     a.packedA = (const half8_t*)state->packed_values;
     a.kidx = state->packed_indices;
-    a.group_ptr = state->panel_ptr;
-    a.indptr = state->args.A_bsr_indptr;
+    a.panel_desc = state->panel_ptr;
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;

@@ -13,9 +13,12 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef int int2_t __attribute__((ext_vector_type(2)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 #define SHFLBW_LDS __attribute__((address_space(3)))
+#define SHFLBW_INLINE_LAMBDA __attribute__((always_inline))
 // read-only data addressed uniformly by a wave: loads through this address space are scalar
 #define SHFLBW_CONST __attribute__((address_space(4)))
 
@@ -58,6 +61,19 @@ __device__ __forceinline__ void global_to_lds_16B(const void* gptr, uint32_t lds
                  :
                  : "v"(gptr), "s"(lds_base)
                  : "m0");
+}
+
+// Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a
+// per-lane 32-bit byte offset: no vector-ALU address arithmetic is needed per copy, which
+// matters because vector-ALU work of one wave competes with the MFMAs of its SIMD neighbour.
+template <int LDS_IMM>
+__device__ __forceinline__ void global_to_lds_16B_sbase(const void* sbase, uint32_t lane_off, uint32_t lds_base)
+{
+    // LDS address = lds_base + LDS_IMM, formed directly in M0
+    asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_off), "s"(sbase), "s"(lds_base), "n"(LDS_IMM)
+                 : "m0", "scc");
 }
 
 // Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids

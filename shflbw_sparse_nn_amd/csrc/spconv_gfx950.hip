@@ -52,11 +52,11 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
     const int n0 = nt * BN;
     const int npix = a.B * a.Ho * a.Wo;
 
-    const int nnz = a.indptr[panel + 1] - a.indptr[panel];
-    const int g0 = a.group_ptr[panel];
+    const int2_t pd = ((const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc)[panel];
+    const int g0 = pd.y;
     const int* __restrict__ kidx = a.kidx + (size_t)g0 * 64;
     const half8_t* __restrict__ pA = a.packedA + (size_t)g0 * (64 * V / 8);
-    const int nsteps = (nnz + 15) >> 4;
+    const int nsteps = pd.x;
     const int ntiles = (nsteps + SPT - 1) / SPT;
 
     // ---- the 8 output pixels this thread loads activations for (same for every pass)

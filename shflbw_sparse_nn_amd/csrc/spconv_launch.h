@@ -11,8 +11,7 @@ struct SpconvLaunchArgs {
     int n_tiles; // pixel tiles, filled by the launcher
     const half8_t* packedA;
     const int* kidx;      // kept k = (r*S + s)*C + c, 64-slot padded per panel
-    const int* group_ptr; // X+1
-    const int* indptr;    // X+1
+    const int* panel_desc; // per panel {k16 steps, first 64-slot group}
     const int* row_ids;   // F, or null
     const half_t* in;     // NHWC
     half_t* out;          // NHWC

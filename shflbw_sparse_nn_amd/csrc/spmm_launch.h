@@ -11,13 +11,14 @@ struct SpmmLaunchArgs {
     int n_tiles; // column tiles, filled by the launcher
     const half8_t* packedA; // private image: A fragments in register order
     const int* kidx;        // private image: kept column ids, 64-slot padded per panel
-    const int* group_ptr;   // X+1, cumulative 64-slot groups
-    const int* indptr;      // X+1, reference-format panel offsets (for the true nnz)
+    const int* kidx_pm;     // same ids, each 64-slot group reordered producer-major: [16p + 4j + r] = [16j + 4p + r]
+    const int* panel_desc;  // private image: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
     const int* row_ids;     // M, or null when rows are not permuted
     const half_t* B;
     const half_t* C;
     half_t* D;
     float alpha, beta;
+    int num_cus; // compute units of the device (persistent kernels size their grid with it)
 };
 
 struct SpmmVariant {

@@ -148,7 +148,9 @@ static void mark_initialized(shflbw_weight* w)
     }
     w->meta_h.clear();
     w->group_ptr.clear();
+    w->panel_desc.clear();
     w->packed_indices.clear();
+    w->packed_indices_pm.clear();
     w->packed_values.clear();
 }
 
@@ -218,8 +220,14 @@ int build_packed_image(shflbw_weight* w)
         int nnz = w->indptr[i + 1] - w->indptr[i];
         w->group_ptr[i + 1] = w->group_ptr[i] + (nnz + 63) / 64;
     }
+    w->panel_desc.assign(2 * (size_t)X, 0);
+    for (int i = 0; i < X; i++) {
+        w->panel_desc[2 * i] = (w->indptr[i + 1] - w->indptr[i] + 15) / 16;
+        w->panel_desc[2 * i + 1] = w->group_ptr[i];
+    }
     const size_t slots = (size_t)w->group_ptr[X] * 64;
     w->packed_indices.assign(slots, 0);
+    w->packed_indices_pm.assign(slots, 0);
     w->packed_values.assign(slots * V, 0);
     for (int i = 0; i < X; i++) {
         const int begin = w->indptr[i], nnz = w->indptr[i + 1] - begin;
@@ -227,6 +235,10 @@ int build_packed_image(shflbw_weight* w)
         const int padded = (w->group_ptr[i + 1] - w->group_ptr[i]) * 64;
         for (int q = 0; q < padded; q++)
             w->packed_indices[slot0 + q] = w->indices[begin + std::min(q, nnz - 1)];
+        for (int q = 0; q < padded; q++) {
+            const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, r = q % 4;
+            w->packed_indices_pm[slot0 + grp * 64 + 16 * p + 4 * j + r] = w->packed_indices[slot0 + q];
+        }
         uint16_t* dst = w->packed_values.data() + slot0 * V;
         const uint16_t* src = w->values.data() + (size_t)begin * V;
         if (V >= 32) {
