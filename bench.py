@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Shfl-BW SpMM, M = K = N = 4096, block size 64, density 0.1, row-permuted
+(BASELINE.json configs[1]) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one launch of the SpMM on device-resident operands (fp16 in, fp32 accumulate, fp16 out).
+Timing follows the reference's benchmark (benchmark/benchmark.spmm.cu:29-50): warm-up launches, then K
+back-to-back launches between two events on the launch stream; mean per launch.  Prints one JSON line:
+effective sparse TFLOP/s (2 * nnzb * V * N / t), the HBM roofline of the kernel, the dense fp16 GEMM of
+the same shape as a reference point, and the CPU oracle timed on the host cores as a baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix-core peak
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=11)
+    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (cfg1 is the graded headline)")
+    ap.add_argument("--variant", type=int, default=-1, help="force a tile variant (default: library choice)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--traffic", default=None,
+                    help="measured HBM bytes per launch (from the rocprofv3 --pmc runs, see profiles/); null if unset")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import shflbw_sparse_nn_amd as S  # raises if the HIP library is missing: there is no fallback
+    from tests import problems as P
+    from tests.gpu_util import to_dev, upload_weight
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    c = P.SPMM_CONFIGS[args.config]
+    M, K, N, V, d = c["M"], c["K"], c["N"], c["V"], c["d"]
+    w = P.make_weight(M, K, V, d, True, 2021, dist=c["a_dist"])
+    B = P.make_dense(K, N, 2021, dist=c["b_dist"])
+    nnzb = w["nnzb"]
+    eff_flops = 2.0 * nnzb * V * N
+    # algorithmic bytes of one launch: A values + (indices, indptr, perm) + B once + D once
+    alg_bytes = nnzb * V * 2 + (nnzb + M // V + 1 + M) * 4 + K * N * 2 + M * N * 2
+
+    mat = upload_weight(w)
+    dB = to_dev(torch, B)
+    dD = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    op = S.SpmmBlockwiseOp(args.variant)
+    st = op.initialize(mat, N, dB.data_ptr(), dD.data_ptr())
+    variant_name = S.spmm_variants(V)[st.variant]
+    stream = torch.cuda.current_stream()
+
+    # correctness gate before any timing: bit-exact against the oracle on the integer twin of the workload
+    from oracle import oracle as O
+    wi = P.make_weight(M, K, V, d, True, 2021, integer=True)
+    Bi = P.make_dense(K, N, 2021, integer=True)
+    mi = upload_weight(wi)
+    dBi = to_dev(torch, Bi)
+    dDi = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    opi = S.SpmmBlockwiseOp(args.variant)
+    opi.initialize(mi, N, dBi.data_ptr(), dDi.data_ptr())
+    opi(stream.cuda_stream)
+    torch.cuda.synchronize()
+    t0 = time.time()
+    ref_i = O.float_to_half(P.spmm_oracle(wi, Bi))
+    t_oracle_all = time.time() - t0
+    if not np.array_equal(dDi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
+        print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
+        sys.exit(1)
+    del mi, dBi, dDi, opi
+
+    # ---- timed region (events on the stream the kernel is launched on)
+    for _ in range(args.warmup):
+        op(stream.cuda_stream)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.time()
+    e0.record(stream)
+    for _ in range(args.steps):
+        op(stream.cuda_stream)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.time() - wall0
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    t = ms_per_step * 1e-3
+    eff_tflops = eff_flops / t / 1e12
+    achieved_gbs = alg_bytes / t / 1e9
+
+    # ---- cold-cache variant: rotate operand sets larger than the 256 MB last-level cache
+    nsets = 5
+    Bs = [dB] + [dB.clone() for _ in range(nsets - 1)]
+    Ds = [dD] + [torch.zeros_like(dD) for _ in range(nsets - 1)]
+    ops = []
+    for i in range(nsets):
+        o = S.SpmmBlockwiseOp(st.variant)
+        o.initialize(mat, N, Bs[i].data_ptr(), Ds[i].data_ptr())
+        ops.append(o)
+    for i in range(nsets):
+        ops[i](stream.cuda_stream)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    for i in range(args.steps):
+        ops[i % nsets](stream.cuda_stream)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    cold_ms = e0.elapsed_time(e1) / args.steps
+    del Bs, Ds, ops
+
+    # ---- dense fp16 GEMM of the same shape (library GEMM behind torch.matmul) as a reference point
+    Ad = torch.randn((M, K), dtype=torch.float16, device="cuda")
+    for _ in range(5):
+        torch.matmul(Ad, dB, out=dD)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    for _ in range(20):
+        torch.matmul(Ad, dB, out=dD)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    dense_ms = e0.elapsed_time(e1) / 20
+
+    # ---- CPU baseline: the oracle (a port of the reference's get_host_reference) on the host cores, on the
+    # same workload; one run with every core, one with a single thread on a 1/8 sample of the row panels
+    cpu = None
+    if not args.no_cpu:
+        threads = O.max_threads()
+        t0 = time.time()
+        P.spmm_oracle(w, B)
+        t_all = time.time() - t0
+        X = M // V
+        sub = dict(w, nrow=(X // 8) * V, indptr=w["indptr"][:X // 8 + 1],
+                   indices=w["indices"][:w["indptr"][X // 8]], values=w["values"][:w["indptr"][X // 8] * V],
+                   row_permute_ids=None)
+        t0 = time.time()
+        P.spmm_oracle(sub, B, nthreads=1)
+        t_one = time.time() - t0
+        sub_flops = 2.0 * int(w["indptr"][X // 8]) * V * N
+        cpu = {"value": round(eff_flops / t_all / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+               "sample": "whole workload (%d panels) with %d threads: %.2f s; single thread on the first %d panels: "
+                         "%.2f s = %.4f TFLOP/s" % (X, threads, t_all, X // 8, t_one, sub_flops / t_one / 1e12)}
+
+    traffic = None if args.traffic is None else float(args.traffic)
+    out = {
+        "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64",
+        "value": round(eff_tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic: seeded Shfl-BW mask + permutation (reference generators, seed 2021), values U[-1,1]",
+        "config": {"workload": "%s: Shfl-BW SpMM M=%d K=%d N=%d, block %d, density %g, row-permuted; nnzb=%d"
+                               % (args.config, M, K, N, V, d, nnzb),
+                   "kernel": variant_name, "timing": "events around %d back-to-back launches, operands resident"
+                                                     % args.steps},
+        "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
+        "dense_equivalent_tflops": round(2.0 * M * N * K / t / 1e12, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "algorithmic_bytes": alg_bytes, "effective_flops": eff_flops},
+        "cold_cache_ms_per_step": round(cold_ms, 6),
+        "dense_gemm": {"what": "torch.matmul fp16 %dx%dx%d (hipBLASLt/rocBLAS)" % (M, N, K),
+                       "ms": round(dense_ms, 6), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 1)},
+        "cpu_baseline": cpu,
+        "wall_s_timed_region": round(wall, 4),
+        "device": S.device_info(),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
