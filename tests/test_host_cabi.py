@@ -133,3 +133,31 @@ def test_variant_table():
         names = S.spmm_variants(V)
         assert len(names) >= 1 and len(set(names)) == len(names)
     assert S.spmm_variants(48) == []
+
+
+def test_static_archive_holds_the_operator_tables():
+    """libblock_sparse.a must define, as unmangled data symbols, the Init/Exec function-pointer variable of
+    every tile configuration named in the table file (the names a user of the reference links against,
+    block_sparse/common/library_util.h:3-9), for SpMM and SpConv alike."""
+    import re
+    import subprocess
+    pkg = os.path.join(ROOT, "shflbw_sparse_nn_amd")
+    archive = os.path.join(pkg, "libblock_sparse.a")
+    assert os.path.exists(archive), "build the library first (__graft_entry__.build())"
+    tuples = []
+    for line in open(os.path.join(pkg, "block_sparse", "common", "library_table.def")):
+        m = re.match(r"SHFLBW_TILE\(([^)]*)\)", line.strip())
+        if m:
+            tuples.append([int(x) for x in m.group(1).split(",")])
+    assert len(tuples) == 83
+    syms = set()
+    for line in subprocess.run(["nm", "--defined-only", archive], stdout=subprocess.PIPE, text=True,
+                               check=True).stdout.splitlines():
+        parts = line.split()
+        if len(parts) == 3 and parts[1] in "DBd":
+            syms.add(parts[2])
+    for t in tuples:
+        tag = "%dx%dx%d_%dx%dx%d_%dx%dx%d_%d" % tuple(t)
+        for kind in ("SpmmBlockwise", "SpconvBlockwise"):
+            for fn in ("Init", "Exec"):
+                assert "%s_%s_%sFn" % (kind, tag, fn) in syms, (kind, tag, fn)
