@@ -76,6 +76,14 @@ __device__ __forceinline__ void global_to_lds_16B_sbase(const void* sbase, uint3
                  : "m0", "scc");
 }
 
+// s_waitcnt on the vector-memory counter that the compiler also treats as a memory fence, for
+// waits that publish LDS contents written by copies the compiler does not know about
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_fence()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 // Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs; this makes consecutive *logical* ids share an XCD (and
 // therefore its L2), so tiles that gather the same activation slab run side by side.

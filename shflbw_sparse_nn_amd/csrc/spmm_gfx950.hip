@@ -280,7 +280,8 @@ struct SpmmWsCfg {
     static constexpr int NB = WN / 32;
     static constexpr int ROWB = BN * 2;
     static constexpr int B_BYTES = KT * ROWB;
-    static constexpr int A_FRAGS = MB;                    // one MFMA k-step per stage
+    static constexpr int KSPS = 1;                        // one MFMA k-step per stage
+    static constexpr int A_FRAGS = MB;
     static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
     static constexpr int RPW = KT / NPROD;                // gathered rows (= copies) per producer and stage
     static constexpr int A_HI = A_FRAGS % NPROD;          // producers [0, A_HI) copy one more A fragment
@@ -337,169 +338,18 @@ struct TileWalker {
     }
 };
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
-__global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
+// Consumer role of the role-split kernels: wave `cw` of NCONS owns the V x WN sub-tile at column
+// cw*WN of every tile of the workgroup.  `Cfg` describes the LDS ring (stage size and count) and the
+// per-wave epilogue area; the barrier protocol is: barrier number t (counted from 0) is passed once
+// stage t of the workgroup's stage stream is complete in LDS; a consumer executes one barrier before
+// its first stage and one more per stage.
+template <typename Cfg, int V, int WN, int NCONS>
+__device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
+                                            int id_end, int S)
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
     constexpr int BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, ROWB = Cfg::ROWB;
-    constexpr int RPW = Cfg::RPW, A_FRAGS = Cfg::A_FRAGS;
     constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
-
-    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N = a.N, X = a.X;
-
-    // ---- this workgroup's tiles: XCD x owns the contiguous id range [x*per, (x+1)*per), ids are
-    // n-tile major (id = nt*X + panel); the S workgroups of the XCD stride through that range.
-    const int T = X * a.n_tiles;
-    const int per = (T + 7) >> 3;
-    const int xcd = blockIdx.x & 7;
-    const int S = gridDim.x >> 3;
-    const int id_first = xcd * per + (blockIdx.x >> 3);
-    const int id_end = min(T, (xcd + 1) * per);
-
-    if (wave >= NCONS) {
-        // =========================== producer ===========================
-        // A wave issues roughly one instruction every four to five cycles, and its vector-ALU
-        // work would compete with the MFMAs of the consumer on the same SIMD; so the per-stage
-        // path below is scalar bookkeeping plus the copies, nothing else, and the scalar state is
-        // kept small enough to stay in registers.
-        const int pw = wave - NCONS;
-        const uint32_t rowbytes = (uint32_t)N * 2;
-        const SHFLBW_CONST int2_t* desc = (const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc;
-        const SHFLBW_CONST int* kpm_all = (const SHFLBW_CONST int*)(uintptr_t)(a.kidx_pm + pw * 16);
-
-        // -- cursor over the non-empty tiles of this workgroup: `cur` is the tile whose stages are
-        // being issued, `nxt` the following non-empty one (descriptor {k16 steps, first group})
-        int id = id_first, idn = id_first;
-        int2_t cur = {0, 0}, nxt = {0, 0};
-        auto find_next = [&]() __attribute__((always_inline)) { // idn, nxt <- next non-empty tile after idn
-            nxt.x = 0;
-            for (idn += S; idn < id_end; idn += S) {
-                nxt = desc[idn % X];
-                if (nxt.x > 0) break;
-            }
-        };
-        idn = id_first - S;
-        find_next();
-        id = idn, cur = nxt; // first non-empty tile (cur.x == 0: none)
-        if (cur.x > 0) find_next();
-
-        int ti = 0;                // stage inside the tile
-        const char* pA = nullptr;  // this wave's A fragment of the stage issued next
-        uint32_t voff[RPW];        // per-lane byte offset inside a B row, one per copy of a stage
-        const uint32_t aoff = lane * 16;
-        auto open_tile = [&]() __attribute__((always_inline)) {
-            ti = 0;
-            const int n0 = (id / X) * BN;
-            pA = (const char*)a.packedA + (size_t)cur.y * (64 * V * 2) + pw * 1024;
-#pragma unroll
-            for (int j = 0; j < RPW; j++) {
-                // copy j fills row pw*RPW + j of the stage; the lane's 16-byte piece lands at
-                // physical position `lane`, i.e. it must fetch logical piece lc of the row
-                const int row = pw * RPW + j;
-                const int lc = ((((lane >> 1) ^ row_xor32(row & 3))) << 1) | (lane & 1);
-                const int col = n0 + lc * 8;
-                voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
-            }
-        };
-
-        // -- kept-column ids: the producer-major copy holds, per 64-slot group, the 16 ids of this
-        // producer contiguously (position 4*j + r: row r of stage j of the group).  `gc*` is the
-        // group being issued, `gn*` the one after it in the stream (possibly the next tile's first),
-        // loaded a whole group ahead.  Named vector values, never an indexable array: a
-        // runtime-indexed array would be demoted to scratch memory, and a scratch load waits for
-        // every copy in flight.
-        int4_t gc0 = {0, 0, 0, 0}, gc1 = gc0, gc2 = gc0, gc3 = gc0;
-        int4_t gn0 = gc0, gn1 = gc0, gn2 = gc0, gn3 = gc0;
-        auto load_group = [&](int first_group, int q) __attribute__((always_inline)) {
-            const SHFLBW_CONST int4_t* g = (const SHFLBW_CONST int4_t*)(kpm_all + ((size_t)first_group + q) * 64);
-            gn0 = g[0], gn1 = g[1], gn2 = g[2], gn3 = g[3];
-        };
-        // called when group q of the current tile becomes the group being issued
-        auto rotate_groups = [&](int q) __attribute__((always_inline)) {
-            gc0 = gn0, gc1 = gn1, gc2 = gn2, gc3 = gn3;
-            if ((q + 1) * 4 < cur.x)
-                load_group(cur.y, q + 1);
-            else if (nxt.x > 0)
-                load_group(nxt.y, 0);
-        };
-
-        uint32_t sb = lds0; // ring slot (LDS byte address) of the next stage to issue
-        uint32_t sbp_b = lds0 + pw * RPW * 1024; // ... where this wave's rows go
-        uint32_t sbp_a = lds0 + pw * 1024;       // ... and its A fragment (plus the B area size)
-        int issued = 0;
-        auto issue_one = [&]() __attribute__((always_inline)) {
-            if (cur.x == 0) return;
-            // sbp = this wave's part of the stage: its B rows start at sbp, its A fragment slots at
-            // sbp + A_BASE (both offsets are compile-time immediates of the copies)
-            constexpr int A_BASE = B_BYTES; // plus pw*1024, folded into sbp_a
-            if (Cfg::A_LO > 0 || pw < Cfg::A_HI) {
-#pragma unroll
-                for (int j = 0; j < Cfg::A_LO + 1; j++)
-                    if (j < Cfg::A_LO || pw < Cfg::A_HI) {
-                        if (j == 0) global_to_lds_16B_sbase<A_BASE>(pA, aoff, sbp_a);
-                        if (j == 1) global_to_lds_16B_sbase<A_BASE + NPROD * 1024>(pA + NPROD * 1024, aoff, sbp_a);
-                    }
-            }
-            const int js = ti & 3;
-            int ks[RPW];
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                int k = gc0[r];
-                k = js == 1 ? gc1[r] : k;
-                k = js == 2 ? gc2[r] : k;
-                k = js == 3 ? gc3[r] : k;
-                ks[r] = k;
-            }
-            static_assert(RPW == 4 && Cfg::A_LO + 1 <= 2, "copies are spelled out for 4 rows and up to 2 fragments");
-            global_to_lds_16B_sbase<0 * 1024>((const char*)a.B + (uint64_t)(uint32_t)ks[0] * rowbytes, voff[0], sbp_b);
-            global_to_lds_16B_sbase<1 * 1024>((const char*)a.B + (uint64_t)(uint32_t)ks[1] * rowbytes, voff[1], sbp_b);
-            global_to_lds_16B_sbase<2 * 1024>((const char*)a.B + (uint64_t)(uint32_t)ks[2] * rowbytes, voff[2], sbp_b);
-            global_to_lds_16B_sbase<3 * 1024>((const char*)a.B + (uint64_t)(uint32_t)ks[3] * rowbytes, voff[3], sbp_b);
-            sbp_b = (sb + STAGE_BYTES == lds0 + Cfg::RING_BYTES) ? sbp_b - (NSTAGE - 1) * STAGE_BYTES : sbp_b + STAGE_BYTES;
-            sbp_a = (sb + STAGE_BYTES == lds0 + Cfg::RING_BYTES) ? sbp_a - (NSTAGE - 1) * STAGE_BYTES : sbp_a + STAGE_BYTES;
-            sb = (sb + STAGE_BYTES == lds0 + Cfg::RING_BYTES) ? lds0 : sb + STAGE_BYTES;
-            pA += A_FRAGS * 1024;
-            issued++;
-            if (++ti == cur.x) { // next tile
-                id = idn, cur = nxt;
-                if (cur.x > 0) {
-                    find_next();
-                    open_tile();
-                    rotate_groups(0);
-                }
-            } else if ((ti & 3) == 0) {
-                rotate_groups(ti >> 2);
-            }
-        };
-
-        if (cur.x > 0) {
-            load_group(cur.y, 0);
-            open_tile();
-            rotate_groups(0);
-        }
-        for (int s = 0; s < NSTAGE - 2; s++) issue_one();
-        // barrier g = -1, 0, 1, ..., issued-1: stage g+1 has landed; afterwards slot of stage g-1 is free
-        for (int g = -1; g < issued; g++) {
-            // copies of at most NSTAGE-3 later stages may stay in flight.  The count uses the
-            // smaller per-stage number of copies (producers that also copy an A fragment issue one
-            // more), which can only make the wait stricter; at the tail fewer stages follow and
-            // everything is drained.
-            if (NSTAGE > 3 && issued - (g + 2) >= NSTAGE - 3)
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * (RPW + Cfg::A_LO)));
-            else
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            wg_barrier();
-            issue_one();
-        }
-        return;
-    }
-
-    // =========================== consumer ===========================
-    const int cw = wave;
     const int li = lane & 15;
     uint32_t boff[NB];
 #pragma unroll
@@ -509,15 +359,19 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
     }
     const uint32_t aoff = (uint32_t)(B_BYTES + lane * 16);
     const uint32_t epi = lds0 + Cfg::RING_BYTES + cw * Cfg::EPI_WAVE_BYTES;
+    constexpr int KSPS = Cfg::KSPS; // k16 steps per LDS stage: rows 16h.. of the B area and A block h belong to step h
+    static_assert(KSPS == 1 || KSPS == 2, "one or two k16 steps per LDS stage");
 
     struct Frags {
         half8_t a[MB], b[NB];
     };
     Frags f0, f1;
-    auto load_frags = [&](uint32_t sbase, Frags& f) __attribute__((always_inline)) {
+    auto load_frags = [&](uint32_t stage_base, int h, Frags& f) __attribute__((always_inline)) {
+        const uint32_t sbase = stage_base + h * (16 * ROWB);
+        const uint32_t abase = stage_base + aoff + h * (MB * 1024);
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
-            f.a[mb] = *(SHFLBW_LDS half8_t*)(uintptr_t)(sbase + aoff + mb * 1024);
+            f.a[mb] = *(SHFLBW_LDS half8_t*)(uintptr_t)(abase + mb * 1024);
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
             const half4_t lo = lds_read_tr16(sbase + boff[nb]);
@@ -569,7 +423,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             wg_barrier();
             // scheduling fences: the reads of the following fragments must be issued before the
             // MFMAs that overlap them, not sunk down to their first use
-            load_frags(sb, nxt);
+            load_frags(sb, 0, nxt);
             __builtin_amdgcn_sched_barrier(0);
             mma(cur);
             __builtin_amdgcn_sched_barrier(0);
@@ -577,10 +431,10 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
 
         if (ntl > 0 && !primed) { // very first stage of the stream
             wg_barrier();
-            load_frags(sb, f0);
+            load_frags(sb, 0, f0);
             primed = true;
         }
-        {
+        if (KSPS == 1) {
             int s = 0;
             for (; s + 1 < ntl; s += 2) {
                 stage(f0, f1);
@@ -589,6 +443,17 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             if (s < ntl) {
                 stage(f0, f1);
                 f0 = f1;
+            }
+        } else {
+            // two k16 steps per LDS stage: the odd step's fragments come from the stage already
+            // present, only the step into the next stage passes a barrier.  A tile with an odd
+            // number of steps computes one padded step (zero A values).
+            for (int p = 0; p < (ntl + 1) >> 1; p++) {
+                load_frags(sb, 1, f1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma(f0);
+                __builtin_amdgcn_sched_barrier(0);
+                stage(f1, f0);
             }
         }
 
@@ -663,12 +528,192 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+__global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    constexpr int BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, ROWB = Cfg::ROWB;
+    constexpr int RPW = Cfg::RPW, A_FRAGS = Cfg::A_FRAGS;
+    constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
+
+    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N = a.N, X = a.X;
+
+    // ---- this workgroup's tiles: XCD x owns the contiguous id range [x*per, (x+1)*per), ids are
+    // n-tile major (id = nt*X + panel); the S workgroups of the XCD stride through that range.
+    const int T = X * a.n_tiles;
+    const int per = (T + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int S = gridDim.x >> 3;
+    const int id_first = xcd * per + (blockIdx.x >> 3);
+    const int id_end = min(T, (xcd + 1) * per);
+
+    if (wave >= NCONS) {
+        // =========================== producer ===========================
+        // A wave issues roughly one instruction every five to six cycles, whatever the kind, and
+        // the workgroup advances one stage per producer round: the round is kept to the copies,
+        // one multiply and one add per gathered row, and a handful of scalar bookkeeping.
+        //  * addresses are a 64-bit base in scalar registers plus a 32-bit per-lane offset; the
+        //    row offset id * row bytes goes into the lane offset (B must be smaller than 4 GiB);
+        //  * the stream is walked group by group (64 slots = up to four stages of one tile); the
+        //    16 ids a producer needs for the next group are fetched by one scalar load at the
+        //    start of the current group and first touched when that group is finished, several
+        //    hundred cycles later, so the full wait a scalar load needs never stalls.
+        const int pw = wave - NCONS;
+        const uint32_t rowbytes = (uint32_t)N * 2;
+        const SHFLBW_CONST int2_t* desc = (const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc;
+        const SHFLBW_CONST int* kpm_all = (const SHFLBW_CONST int*)(uintptr_t)(a.kidx_pm + pw * 16);
+        constexpr int OPS = RPW + Cfg::A_LO; // copies per stage that every producer issues at least
+        static_assert(RPW == 4 && A_FRAGS <= 2 * NPROD, "the stage is spelled out for 4 rows and up to 2 fragments per producer");
+
+        // -- cursor over the non-empty tiles of this workgroup
+        int id = id_first, idn = id_first;
+        int2_t cur = {0, 0}, nxt = {0, 0};
+        auto find_next = [&]() __attribute__((always_inline)) { // idn, nxt <- next non-empty tile after idn
+            nxt.x = 0;
+            for (idn += S; idn < id_end; idn += S) {
+                nxt = desc[idn % X];
+                if (nxt.x > 0) break;
+            }
+        };
+        idn = id_first - S;
+        find_next();
+        id = idn, cur = nxt; // first non-empty tile (cur.x == 0: none)
+        if (cur.x == 0) return; // no stage at all: the consumers pass no barrier either
+        find_next();
+
+        // -- per-tile lane offsets: copy j of a stage fills row pw*4 + j; the lane's 16-byte piece
+        // lands at physical position `lane`, so it fetches logical piece lc of the row
+        uint32_t voff[RPW];
+        uint32_t va = 0;             // lane offset of this wave's A fragment of the next stage
+        const char* tileA = nullptr; // A fragments of the current tile
+        auto open_tile = [&]() __attribute__((always_inline)) {
+            const int n0 = (id / X) * BN;
+            tileA = (const char*)a.packedA + (size_t)cur.y * (64 * V * 2);
+            va = pw * 1024 + lane * 16;
+#pragma unroll
+            for (int j = 0; j < RPW; j++) {
+                const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
+                const int col = n0 + lc * 8;
+                voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
+            }
+        };
+
+        // -- ring position of the next stage: LDS address of this wave's four rows
+        uint32_t sbp = lds0 + pw * RPW * 1024;
+        const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's first A fragment slot relative to sbp
+        int issued = 0;
+        // one stage: optional wait + barrier, then the copies
+        auto stage = [&](int k0, int k1, int k2, int k3) __attribute__((always_inline)) {
+            if (issued >= NSTAGE - 2) {
+                // barrier g = issued - (NSTAGE-1): stage g+1 must have landed, NSTAGE-3 younger
+                // stages may stay in flight
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * OPS));
+                wg_barrier();
+            }
+            uint32_t t0, t1, t2, t3, v0, v1, v2, v3;
+            asm volatile("s_mul_i32 %[t0], %[k0], %[rb]\n\t"
+                         "s_mul_i32 %[t1], %[k1], %[rb]\n\t"
+                         "s_mul_i32 %[t2], %[k2], %[rb]\n\t"
+                         "s_mul_i32 %[t3], %[k3], %[rb]\n\t"
+                         "s_mov_b32 m0, %[sbp]\n\t"
+                         "v_add_u32 %[v0], %[t0], %[l0]\n\t"
+                         "global_load_lds_dwordx4 %[v0], %[B]\n\t"
+                         "s_add_i32 m0, %[sbp], 0x400\n\t"
+                         "v_add_u32 %[v1], %[t1], %[l1]\n\t"
+                         "global_load_lds_dwordx4 %[v1], %[B]\n\t"
+                         "s_add_i32 m0, %[sbp], 0x800\n\t"
+                         "v_add_u32 %[v2], %[t2], %[l2]\n\t"
+                         "global_load_lds_dwordx4 %[v2], %[B]\n\t"
+                         "s_add_i32 m0, %[sbp], 0xc00\n\t"
+                         "v_add_u32 %[v3], %[t3], %[l3]\n\t"
+                         "global_load_lds_dwordx4 %[v3], %[B]"
+                         : [t0] "=&s"(t0), [t1] "=&s"(t1), [t2] "=&s"(t2), [t3] "=&s"(t3), [v0] "=&v"(v0),
+                           [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3)
+                         : [k0] "s"(k0), [k1] "s"(k1), [k2] "s"(k2), [k3] "s"(k3), [rb] "s"(rowbytes),
+                           [l0] "v"(voff[0]), [l1] "v"(voff[1]), [l2] "v"(voff[2]), [l3] "v"(voff[3]),
+                           [B] "s"(a.B), [sbp] "s"(sbp)
+                         : "m0", "scc");
+            if (Cfg::A_LO > 0 || pw < Cfg::A_HI) {
+                asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
+                             "s_nop 0\n\t"
+                             "global_load_lds_dwordx4 %[va], %[A]"
+                             :
+                             : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
+                             : "m0", "scc");
+                if (Cfg::A_LO > 0 && pw < Cfg::A_HI) // a second fragment, NPROD fragments further on
+                    asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
+                                 "s_nop 0\n\t"
+                                 "global_load_lds_dwordx4 %[va], %[A]"
+                                 :
+                                 : [sbp] "s"(sbp), [arel] "s"(a_rel + NPROD * 1024), [va] "v"(va + NPROD * 1024),
+                                   [A] "s"(tileA)
+                                 : "m0", "scc");
+            }
+            va += A_FRAGS * 1024;
+            sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
+                                                                                   : sbp + STAGE_BYTES;
+            issued++;
+        };
+
+        // -- groups: gc* = ids of the group being issued (position 4*j + r of the producer-major
+        // copy: row r of stage j), gn* = ids of the group after it in the stream
+        auto load_group = [&](int group) __attribute__((always_inline)) {
+            return (const SHFLBW_CONST int4_t*)(kpm_all + (size_t)group * 64);
+        };
+        const SHFLBW_CONST int4_t* g = load_group(cur.y);
+        int4_t gc0 = g[0], gc1 = g[1], gc2 = g[2], gc3 = g[3];
+        open_tile();
+        while (true) {
+            const int ngroups = (cur.x + 3) >> 2;
+            for (int q = 0; q < ngroups; q++) {
+                const int n = min(4, cur.x - 4 * q);
+                // the group that follows in the stream; at the very end simply this one again
+                int gnext = cur.y + q + 1;
+                if (q + 1 == ngroups) gnext = nxt.x > 0 ? nxt.y : cur.y + q;
+                const SHFLBW_CONST int4_t* gp = load_group(gnext);
+                const int4_t gn0 = gp[0], gn1 = gp[1], gn2 = gp[2], gn3 = gp[3];
+                stage(gc0.x, gc0.y, gc0.z, gc0.w);
+                if (n > 1) stage(gc1.x, gc1.y, gc1.z, gc1.w);
+                if (n > 2) stage(gc2.x, gc2.y, gc2.z, gc2.w);
+                if (n > 3) stage(gc3.x, gc3.y, gc3.z, gc3.w);
+                gc0 = gn0, gc1 = gn1, gc2 = gn2, gc3 = gn3;
+            }
+            if (nxt.x == 0) break;
+            id = idn, cur = nxt;
+            find_next();
+            open_tile();
+        }
+        // -- tail: `issued` stages are out, barriers g = issued-(NSTAGE-1) ... issued-1 remain
+        for (int g2 = max(issued - (NSTAGE - 1), -1); g2 < issued; g2++) {
+            const int younger = issued - g2 - 2; // stages issued after stage g2+1, which must have landed
+            if (NSTAGE > 5 && younger >= 3)
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * OPS));
+            else if (NSTAGE > 4 && younger == 2)
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * OPS));
+            else if (NSTAGE > 3 && younger == 1)
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(1 * OPS));
+            else
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            wg_barrier();
+        }
+        return;
+    }
+
+    ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
     SpmmLaunchArgs b = a;
     b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
     const int T = a.X * b.n_tiles;
+    // the gather addresses rows of B with 32-bit byte offsets
+    if ((unsigned long long)a.K * (unsigned long long)a.N * 2ull > 0xffffffffull) return hipErrorInvalidValue;
     // one persistent workgroup per compute unit; fewer when there are fewer tiles (multiple of 8 XCDs)
     int grid = a.num_cus > 0 ? a.num_cus : 256;
     grid = (grid / 8) * 8;
@@ -686,6 +731,253 @@ static hipError_t prepare_ws()
     return hipFuncSetAttribute((const void*)spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
 }
+
+// =======================================================================================
+// Register-staged variant of the role-split kernel.
+//
+// The gather has a latency of one to two microseconds (part of every stage misses the L2), so
+// keeping the matrix cores fed needs on the order of ten stages in flight per compute unit -
+// more bytes than the LDS can hold.  Here the producers therefore gather with ordinary vector
+// loads into a ring of registers DEPTH stages deep (a producer wave has 64 KiB of registers and
+// nothing else to keep in them) and move a stage into a short LDS ring only when it has
+// arrived.  All loads are visible to the compiler, which counts the in-order vector-memory
+// counter exactly; the kept-column ids ride the same counter (one 16-byte uniform load per
+// stage and producer, fetched a further DEPTH stages ahead).
+// LDS ring: stage t lives in slot t % 3.  A consumer has finished reading stage t when it
+// arrives at barrier t+2, the producers write stage t after barrier t-1: three slots suffice.
+// =======================================================================================
+template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
+struct SpmmRsCfg {
+    static constexpr int NSTAGE = 3;
+    static constexpr int KSPS = KT / 16;                  // MFMA k-steps per LDS stage
+    static constexpr int BN = WN * NCONS;
+    static constexpr int MB = V / 32;
+    static constexpr int NB = WN / 32;
+    static constexpr int ROWB = BN * 2;
+    static constexpr int B_BYTES = KT * ROWB;
+    static constexpr int A_FRAGS = MB;                    // per k-step
+    static constexpr int A_BYTES = KSPS * A_FRAGS * 1024; // per stage, contiguous in memory and in LDS
+    static constexpr int STAGE_BYTES = B_BYTES + A_BYTES;
+    static constexpr int RPW = KT / NPROD;
+    static constexpr int APL = A_BYTES / (NPROD * 64);    // A bytes per producer lane and stage
+    static constexpr int LOADS = RPW + 1 + RPW / 4;       // vector loads per producer and stage
+    static constexpr int EPI_ROWB = WN * 2 + 16;
+    static constexpr int EPI_WAVE_BYTES = 32 * EPI_ROWB;
+    static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+    static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
+    static constexpr int THREADS = (NCONS + NPROD) * 64;
+    static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
+    static_assert(BN == 512, "one gathered row is one 1 KiB wave access");
+    static_assert((KT == 16 || KT == 32) && NPROD == 4, "four producers, one or two k16 steps per stage");
+    static_assert(APL == 4 || APL == 8 || APL == 16, "the A block of a stage splits evenly over the producer lanes");
+    static_assert(DEPTH * LOADS < 64, "vmcnt is a 6-bit counter");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
+};
+
+// Cursor over the stages of a workgroup's non-empty tiles, in stream order.  Past the last stage
+// it stays on the last stage (`done` set), so that addresses derived from it remain valid: the
+// producers' pipeline issues a fixed number of loads per step and simply re-reads that stage.
+struct StageCursor {
+    int id, idn, end, S, X; // current tile, next non-empty tile, range end, stride, panels
+    int2_t cur, nxt;        // descriptors {k16 steps, first 64-slot group}; cur.x == 0: no stage at all
+    int ti;                 // stage inside the current tile
+    int kshift;             // log2 of the k16 steps per stage
+    bool done;
+    __device__ __forceinline__ int stages() const { return (cur.x + (1 << kshift) - 1) >> kshift; }
+    const SHFLBW_CONST int2_t* desc;
+    __device__ __forceinline__ void find_next()
+    {
+        nxt.x = 0;
+        for (idn += S; idn < end; idn += S) {
+            nxt = desc[idn % X];
+            if (nxt.x > 0) break;
+        }
+    }
+    __device__ __forceinline__ void init(const int* d, int first, int end_, int S_, int X_, int kshift_)
+    {
+        desc = (const SHFLBW_CONST int2_t*)(uintptr_t)d;
+        end = end_, S = S_, X = X_, ti = 0, kshift = kshift_;
+        idn = first - S;
+        nxt.x = 0, nxt.y = 0;
+        find_next();
+        id = idn, cur = nxt;
+        done = cur.x == 0;
+        if (!done) find_next();
+    }
+    // returns true when the step entered a new tile
+    __device__ __forceinline__ bool advance()
+    {
+        if (ti + 1 < stages()) {
+            ti++;
+            return false;
+        }
+        if (nxt.x == 0) {
+            done = true;
+            return false;
+        }
+        ti = 0, id = idn, cur = nxt;
+        find_next();
+        return true;
+    }
+};
+
+template <int BYTES> struct LaneChunk;
+template <> struct LaneChunk<4> { typedef int type; };
+template <> struct LaneChunk<8> { typedef int2_t type; };
+template <> struct LaneChunk<16> { typedef int4_t type; };
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
+__global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_rs_kernel(SpmmLaunchArgs a)
+{
+    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
+    constexpr int BN = Cfg::BN, RPW = Cfg::RPW, APL = Cfg::APL;
+    constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES, A_BYTES = Cfg::A_BYTES;
+    // the A block of a stage is moved in equal shares by all producers, so every producer issues
+    // exactly the same loads per stage
+    typedef typename LaneChunk<APL>::type achunk_t;
+
+    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N = a.N, X = a.X;
+
+    // same tile -> workgroup map as the copy-based kernel: XCD x owns a contiguous id range
+    const int T = X * a.n_tiles;
+    const int per = (T + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int S = gridDim.x >> 3;
+    const int id_first = xcd * per + (blockIdx.x >> 3);
+    const int id_end = min(T, (xcd + 1) * per);
+
+    if (wave < NCONS) {
+        ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
+        return;
+    }
+
+    // =========================== producer ===========================
+    // Everything on the stage cadence is unconditional: the compiler derives exact vmcnt waits only
+    // when every path through the loop issues the same loads in the same order.
+    const int pw = wave - NCONS;
+    // a zero the compiler cannot see through: added to wave-uniform addresses so that the id loads
+    // stay vector loads (a scalar load would need a full wait and has no place in this pipeline)
+    uint32_t vzero = 0;
+    asm volatile("" : "+v"(vzero));
+
+    StageCursor ic, rc; // the id-load cursor runs DEPTH stages ahead of the row-load cursor
+    ic.init(a.panel_desc, id_first, id_end, S, X, Cfg::KSPS == 2 ? 1 : 0);
+    if (ic.done) return; // no stage: the consumers execute no barrier either
+    rc = ic;
+
+    half8_t rb[DEPTH][RPW]; // gathered rows in flight
+    achunk_t ra[DEPTH];     // A shares in flight
+    int4_t ri[DEPTH][RPW / 4]; // ids of the stage whose rows are requested next from this ring position
+
+    auto load_ids = [&](int4_t (&dst)[RPW / 4]) __attribute__((always_inline)) {
+        const int* p = a.kidx + ((size_t)ic.cur.y * 64 + ic.ti * KT + pw * RPW);
+#pragma unroll
+        for (int q = 0; q < RPW / 4; q++) dst[q] = *(const int4_t*)((const char*)p + q * 16 + vzero);
+        ic.advance();
+    };
+
+    // per-tile state of the row cursor
+    uint32_t voff[4];                                     // lane byte offsets inside a B row, by row % 4
+    const uint32_t aoff = pw * (64 * APL) + lane * APL;   // lane byte offset inside the A block of a stage
+    const char* tileA = nullptr;                          // A blocks of the current tile
+    auto open_tile = [&]() __attribute__((always_inline)) {
+        const int n0 = (rc.id / X) * BN;
+        tileA = (const char*)a.packedA + (size_t)rc.cur.y * (64 * V * 2);
+#pragma unroll
+        for (int j = 0; j < 4; j++) { // RPW is a multiple of 4: row pw*RPW + j has swizzle key j % 4
+            const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
+            const int col = n0 + lc * 8;
+            voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
+        }
+    };
+    const size_t rowbytes = (size_t)N * 2;
+    int real = 0; // stages of the stream whose rows have been requested
+    auto load_rows = [&](const int4_t (&ids)[RPW / 4], half8_t (&dstb)[RPW], achunk_t& dsta) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            const int k = __builtin_amdgcn_readfirstlane(ids[r / 4][r % 4]);
+            dstb[r] = *(const half8_t*)((const char*)a.B + (size_t)(uint32_t)k * rowbytes + voff[r & 3]);
+        }
+        dsta = *(const achunk_t*)(tileA + (size_t)rc.ti * A_BYTES + aoff);
+        if (!rc.done) {
+            real++;
+            if (rc.advance()) open_tile();
+        }
+    };
+
+    // ---- prologue: ids of the first DEPTH stages, their rows, and the ids of the DEPTH after them
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) load_ids(ri[j]);
+    open_tile();
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) {
+        load_rows(ri[j], rb[j], ra[j]);
+        load_ids(ri[j]);
+    }
+
+    // ---- stage t: move it from the registers into LDS slot t % 3, request stage t + DEPTH into the
+    // same registers, pass barrier t
+    const uint32_t wr_b = lds0 + pw * RPW * 1024 + lane * 16;
+    const uint32_t wr_a = lds0 + B_BYTES + aoff;
+    uint32_t slot = 0; // byte offset of the LDS slot of the stage moved next
+    auto move_stage = [&](half8_t (&srcb)[RPW], achunk_t& srca, int4_t (&ids)[RPW / 4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < RPW; r++) *(SHFLBW_LDS half8_t*)(uintptr_t)(wr_b + slot + r * 1024) = srcb[r];
+        *(SHFLBW_LDS achunk_t*)(uintptr_t)(wr_a + slot) = srca;
+        slot = (slot + STAGE_BYTES == Cfg::RING_BYTES) ? 0 : slot + STAGE_BYTES;
+        load_rows(ids, srcb, srca);
+        load_ids(ids);
+        __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the LDS writes of this stage are done
+        wg_barrier();
+    };
+    int t = 0;
+    // steady state: DEPTH real stages are resident in the ring
+    while (real - t >= DEPTH) {
+#pragma unroll
+        for (int j = 0; j < DEPTH; j++) move_stage(rb[j], ra[j], ri[j]);
+        t += DEPTH;
+    }
+    // tail of the stream: fewer than DEPTH stages left, ring positions 0 .. real - t - 1
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++)
+        if (t + j < real) move_stage(rb[j], ra[j], ri[j]);
+    wg_barrier(); // the consumers' last stage passes one more barrier
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
+static hipError_t launch_rs(const SpmmLaunchArgs& a, hipStream_t stream)
+{
+    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
+    SpmmLaunchArgs b = a;
+    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    const int T = a.X * b.n_tiles;
+    int grid = a.num_cus > 0 ? a.num_cus : 256;
+    grid = (grid / 8) * 8;
+    const int need = ((T + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL((spmm_shflbw_rs_kernel<V, WN, NCONS, NPROD, KT, DEPTH>), dim3(grid), dim3(Cfg::THREADS),
+                       Cfg::LDS_BYTES, stream, b);
+    return hipGetLastError();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
+static hipError_t prepare_rs()
+{
+    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
+    return hipFuncSetAttribute((const void*)spmm_shflbw_rs_kernel<V, WN, NCONS, NPROD, KT, DEPTH>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+}
+
+#define SHFLBW_RS_VARIANT(V, WN, NC, NP, KT, D)                                                              \
+    {                                                                                                        \
+        V, WN* NC, (NC + NP) * 64, SpmmRsCfg<V, WN, NC, NP, KT, D>::LDS_BYTES,                                \
+            "rs" #V "x" #WN "x" #NC "c" #NP "p_k" #KT "_d" #D, &launch_rs<V, WN, NC, NP, KT, D>,             \
+            &prepare_rs<V, WN, NC, NP, KT, D>                                                                 \
+    }
 
 #define SHFLBW_WS_VARIANT(V, WN, NC, NP, KT, NS)                                                             \
     {                                                                                                        \
@@ -728,6 +1020,10 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 4),
+    SHFLBW_RS_VARIANT(64, 128, 4, 4, 32, 4),
+    SHFLBW_RS_VARIANT(64, 128, 4, 4, 32, 3),
+    SHFLBW_RS_VARIANT(64, 128, 4, 4, 16, 8),
+    SHFLBW_RS_VARIANT(64, 128, 4, 4, 16, 4),
     SHFLBW_VARIANT(64, 64, 4, 32, 3),
     SHFLBW_VARIANT(64, 64, 4, 32, 2),
     SHFLBW_VARIANT(64, 64, 4, 16, 4),
