@@ -280,22 +280,26 @@ struct SpmmWsCfg {
     static constexpr int NB = WN / 32;
     static constexpr int ROWB = BN * 2;
     static constexpr int B_BYTES = KT * ROWB;
-    static constexpr int KSPS = 1;                        // one MFMA k-step per stage
-    static constexpr int A_FRAGS = MB;
+    static constexpr int KSPS = KT / 16;                  // MFMA k-steps per stage
+    static constexpr int A_FRAGS = KSPS * MB;             // 1 KiB fragments per stage, contiguous in memory and LDS
     static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
     static constexpr int RPW = KT / NPROD;                // gathered rows (= copies) per producer and stage
     static constexpr int A_HI = A_FRAGS % NPROD;          // producers [0, A_HI) copy one more A fragment
     static constexpr int A_LO = A_FRAGS / NPROD;
-    static constexpr int EPI_ROWB = WN * 2 + 16;
-    static constexpr int EPI_WAVE_BYTES = 32 * EPI_ROWB;  // one 32-row block of a consumer's sub-tile
+    static constexpr int OPS = RPW + A_LO;                // copies per stage every producer issues at least
+    static constexpr int EPI_ROWB = 32 * 2 + 16;
+    static constexpr int EPI_ROWS = NCONS > 4 ? 16 : 32;  // rows of a 32 x 32 accumulator block staged at a time
+    static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
     static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
     static_assert(BN == 512, "one gathered row is exactly one 1 KiB copy instruction");
-    static_assert(KT == 16 && NPROD == 4, "the producer-major index copy is laid out for 4 producers x 4 rows x 4 stages");
+    static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
+    static_assert(A_LO <= 1 && (A_LO == 0 || A_HI == 0), "at most one A fragment per producer and stage");
+    static_assert(THREADS <= 1024, "workgroup size limit");
     static_assert(NSTAGE >= 3, "one stage computed, one landed, one in flight");
-    static_assert((NSTAGE - 3) * (RPW + A_LO + 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert((NSTAGE - 3) * OPS < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 };
 
@@ -457,53 +461,63 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             }
         }
 
-        // ---- epilogue of this wave's V x WN sub-tile, one 32-row block at a time: accumulators
-        // -> fp16 (one rounding) -> private LDS area (a lane holds 4 consecutive columns of one
-        // row per 8-byte write) -> 16-byte pieces of whole row segments -> scattered rows of D
-        constexpr int PR = WN / 8;       // 16-byte pieces per row of the sub-tile
-        constexpr int RPS = 64 / PR;     // rows per store instruction
-        constexpr int NIT = 32 / RPS;
+        // ---- epilogue of this wave's V x WN sub-tile, one 32 x 32 accumulator block at a time:
+        // fp16 (one rounding) -> private LDS area (a lane holds 4 consecutive columns of one row
+        // per 8-byte write) -> 16-byte pieces of 64-byte row segments -> scattered rows of D.  The
+        // staging area is small on purpose: the LDS belongs to the stage ring.
+        constexpr int PR = 4;                 // 16-byte pieces per 32-column row segment
+        constexpr int RPS = 64 / PR;          // rows per store instruction
+        constexpr int ER = Cfg::EPI_ROWS;     // rows staged at a time: 32 (whole block) or 16 (half, by lanes)
+        constexpr int NIT = ER / RPS;
         const int pc = lane % PR;
-        const int col = n0 + cw * WN + pc * 8;
-        const bool col_ok = col < N;
-        const uint32_t wr = epi + (lane & 31) * Cfg::EPI_ROWB + (lane >> 5) * 8;
+        const int col0 = n0 + cw * WN + pc * 8;
+        const uint32_t wr = epi + (lane & (ER - 1)) * Cfg::EPI_ROWB + (lane >> 5) * 8;
         const uint32_t rd = epi + (lane / PR) * Cfg::EPI_ROWB + pc * 16;
         // specialised on "alpha == 1" and "beta == 0" so that the common path has no branch (a
         // branch per piece would put a full wait at every join)
         auto epi_block = [&](int mb, auto scale, auto add_c) __attribute__((always_inline)) {
             constexpr bool SCALE = decltype(scale)::value, ADDC = decltype(add_c)::value;
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++)
+            for (int hh = 0; hh < 32 / ER; hh++) {
+                size_t roff[NIT]; // element offset of the lane's output row, without the column
 #pragma unroll
-                for (int ig = 0; ig < 4; ig++) {
-                    half4_t h;
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        h[e] = (half_t)(SCALE ? acc[mb][nb][ig * 4 + e] * alpha : acc[mb][nb][ig * 4 + e]);
-                    *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + (nb * 32 + ig * 8) * 2) = h;
+                for (int it = 0; it < NIT; it++) {
+                    const int rr = mb * 32 + hh * ER + it * RPS + lane / PR;
+                    roff[it] = (size_t)__shfl(rid[rr >> 6], rr & 63) * N;
                 }
-            // all loads (LDS pieces, C when used), then all stores: the vector-memory counter is
-            // in-order, a load issued behind a store would wait for the store to complete
-            half8_t v[NIT], c[NIT];
-            size_t off[NIT];
 #pragma unroll
-            for (int it = 0; it < NIT; it++) {
-                v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * RPS * Cfg::EPI_ROWB);
-                const int rr = mb * 32 + it * RPS + lane / PR;
-                const int orow = __shfl(rid[rr >> 6], rr & 63);
-                off[it] = (size_t)orow * N + col;
-            }
-            if (col_ok) {
-                if (ADDC) {
+                for (int nb = 0; nb < NB; nb++) {
+                    if (ER == 32 || ((lane >> 4) & 1) == hh) { // a lane holds row lane % 32 of the block
 #pragma unroll
-                    for (int it = 0; it < NIT; it++) c[it] = *(const half8_t*)(a.C + off[it]);
+                        for (int ig = 0; ig < 4; ig++) {
+                            half4_t h;
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                h[e] = (half_t)(SCALE ? acc[mb][nb][ig * 4 + e] * alpha : acc[mb][nb][ig * 4 + e]);
+                            *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + ig * 16) = h;
+                        }
+                    }
+                    // all loads (LDS pieces, C when used), then all stores: the vector-memory
+                    // counter is in-order, a load issued behind a store would wait for the store
+                    half8_t v[NIT], c[NIT];
 #pragma unroll
                     for (int it = 0; it < NIT; it++)
+                        v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * RPS * Cfg::EPI_ROWB);
+                    const int col = col0 + nb * 32;
+                    if (col < N) {
+                        if (ADDC) {
 #pragma unroll
-                        for (int e = 0; e < 8; e++) v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
+                            for (int it = 0; it < NIT; it++) c[it] = *(const half8_t*)(a.C + roff[it] + col);
+#pragma unroll
+                            for (int it = 0; it < NIT; it++)
+#pragma unroll
+                                for (int e = 0; e < 8; e++)
+                                    v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
+                        }
+#pragma unroll
+                        for (int it = 0; it < NIT; it++) *(half8_t*)(a.D + roff[it] + col) = v[it];
+                    }
                 }
-#pragma unroll
-                for (int it = 0; it < NIT; it++) *(half8_t*)(a.D + off[it]) = v[it];
             }
         };
         // The row ids were loaded at the start of the tile.  Consume them here once: the wait the
@@ -527,12 +541,45 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
     }
 }
 
+// Four gathered rows of B (ids k, wave-uniform) into four consecutive 1 KiB LDS rows starting
+// ROW0 rows after sbp: per row one scalar multiply (id * row bytes fits 32 bits), one vector add
+// onto the lane's column offset, and the copy; the add doubles as the wait state the copy needs
+// after the write of M0.
+template <int ROW0>
+__device__ __forceinline__ void gather_rows4(int4_t k, uint32_t rowbytes, const uint32_t (&voff)[4], const void* B,
+                                             uint32_t sbp)
+{
+    constexpr int O = ROW0 * 1024;
+    uint32_t t0, t1, t2, t3, v0, v1, v2, v3;
+    asm volatile("s_mul_i32 %[t0], %[k0], %[rb]\n\t"
+                 "s_mul_i32 %[t1], %[k1], %[rb]\n\t"
+                 "s_mul_i32 %[t2], %[k2], %[rb]\n\t"
+                 "s_mul_i32 %[t3], %[k3], %[rb]\n\t"
+                 "s_add_i32 m0, %[sbp], %[o0]\n\t"
+                 "v_add_u32 %[v0], %[t0], %[l0]\n\t"
+                 "global_load_lds_dwordx4 %[v0], %[B]\n\t"
+                 "s_add_i32 m0, %[sbp], %[o1]\n\t"
+                 "v_add_u32 %[v1], %[t1], %[l1]\n\t"
+                 "global_load_lds_dwordx4 %[v1], %[B]\n\t"
+                 "s_add_i32 m0, %[sbp], %[o2]\n\t"
+                 "v_add_u32 %[v2], %[t2], %[l2]\n\t"
+                 "global_load_lds_dwordx4 %[v2], %[B]\n\t"
+                 "s_add_i32 m0, %[sbp], %[o3]\n\t"
+                 "v_add_u32 %[v3], %[t3], %[l3]\n\t"
+                 "global_load_lds_dwordx4 %[v3], %[B]"
+                 : [t0] "=&s"(t0), [t1] "=&s"(t1), [t2] "=&s"(t2), [t3] "=&s"(t3), [v0] "=&v"(v0), [v1] "=&v"(v1),
+                   [v2] "=&v"(v2), [v3] "=&v"(v3)
+                 : [k0] "s"(k.x), [k1] "s"(k.y), [k2] "s"(k.z), [k3] "s"(k.w), [rb] "s"(rowbytes), [l0] "v"(voff[0]),
+                   [l1] "v"(voff[1]), [l2] "v"(voff[2]), [l3] "v"(voff[3]), [B] "s"(B), [sbp] "s"(sbp), [o0] "n"(O),
+                   [o1] "n"(O + 0x400), [o2] "n"(O + 0x800), [o3] "n"(O + 0xc00)
+                 : "m0", "scc");
+}
+
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
-    constexpr int BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, ROWB = Cfg::ROWB;
-    constexpr int RPW = Cfg::RPW, A_FRAGS = Cfg::A_FRAGS;
+    constexpr int BN = Cfg::BN, RPW = Cfg::RPW;
     constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
 
     extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
@@ -564,9 +611,19 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         const int pw = wave - NCONS;
         const uint32_t rowbytes = (uint32_t)N * 2;
         const SHFLBW_CONST int2_t* desc = (const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc;
-        const SHFLBW_CONST int* kpm_all = (const SHFLBW_CONST int*)(uintptr_t)(a.kidx_pm + pw * 16);
-        constexpr int OPS = RPW + Cfg::A_LO; // copies per stage that every producer issues at least
-        static_assert(RPW == 4 && A_FRAGS <= 2 * NPROD, "the stage is spelled out for 4 rows and up to 2 fragments per producer");
+        constexpr int OPS = Cfg::OPS, KSPS = Cfg::KSPS;
+        constexpr int NSG = 64 / KT; // stages per group
+        // ids of a group for this producer, as int4 number q.  Four rows per producer and stage:
+        // stage j uses int4 j - with 16-row stages from the producer-major copy [16 pw + 4 j + r],
+        // with 32-row stages (8 producers) from slots 32 j + 4 pw + r of the slot-ordered array.
+        // Eight rows per producer and stage (32-row stages, 4 producers): stage j uses int4 2j and
+        // 2j+1, slots 32 j + 8 pw + r.
+        auto group_ptr = [&](int group, int q) __attribute__((always_inline)) {
+            const int* base = KT == 16   ? a.kidx_pm + (size_t)group * 64 + pw * 16 + q * 4
+                              : RPW == 8 ? a.kidx + (size_t)group * 64 + (q >> 1) * 32 + pw * 8 + (q & 1) * 4
+                                         : a.kidx + (size_t)group * 64 + (q & 1) * 32 + pw * 4;
+            return (const SHFLBW_CONST int4_t*)(uintptr_t)base;
+        };
 
         // -- cursor over the non-empty tiles of this workgroup
         int id = id_first, idn = id_first;
@@ -582,11 +639,11 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         find_next();
         id = idn, cur = nxt; // first non-empty tile (cur.x == 0: none)
         if (cur.x == 0) return; // no stage at all: the consumers pass no barrier either
-        find_next();
+        bool have_next = false;   // `nxt` describes the tile after `cur`
 
-        // -- per-tile lane offsets: copy j of a stage fills row pw*4 + j; the lane's 16-byte piece
-        // lands at physical position `lane`, so it fetches logical piece lc of the row
-        uint32_t voff[RPW];
+        // -- per-tile lane offsets: copy j of a stage fills row pw*RPW + j (swizzle key j % 4); the
+        // lane's 16-byte piece lands at physical position `lane`, so it fetches logical piece lc
+        uint32_t voff[4];
         uint32_t va = 0;             // lane offset of this wave's A fragment of the next stage
         const char* tileA = nullptr; // A fragments of the current tile
         auto open_tile = [&]() __attribute__((always_inline)) {
@@ -594,91 +651,79 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             tileA = (const char*)a.packedA + (size_t)cur.y * (64 * V * 2);
             va = pw * 1024 + lane * 16;
 #pragma unroll
-            for (int j = 0; j < RPW; j++) {
+            for (int j = 0; j < 4; j++) {
                 const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
                 const int col = n0 + lc * 8;
                 voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
             }
         };
 
-        // -- ring position of the next stage: LDS address of this wave's four rows
+        // -- ring position of the next stage: LDS address of this wave's rows
         uint32_t sbp = lds0 + pw * RPW * 1024;
-        const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's first A fragment slot relative to sbp
+        const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's A fragment slot relative to sbp
         int issued = 0;
         // one stage: optional wait + barrier, then the copies
-        auto stage = [&](int k0, int k1, int k2, int k3) __attribute__((always_inline)) {
+        auto stage = [&](int4_t ka, int4_t kb) __attribute__((always_inline)) {
             if (issued >= NSTAGE - 2) {
                 // barrier g = issued - (NSTAGE-1): stage g+1 must have landed, NSTAGE-3 younger
                 // stages may stay in flight
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * OPS));
                 wg_barrier();
             }
-            uint32_t t0, t1, t2, t3, v0, v1, v2, v3;
-            asm volatile("s_mul_i32 %[t0], %[k0], %[rb]\n\t"
-                         "s_mul_i32 %[t1], %[k1], %[rb]\n\t"
-                         "s_mul_i32 %[t2], %[k2], %[rb]\n\t"
-                         "s_mul_i32 %[t3], %[k3], %[rb]\n\t"
-                         "s_mov_b32 m0, %[sbp]\n\t"
-                         "v_add_u32 %[v0], %[t0], %[l0]\n\t"
-                         "global_load_lds_dwordx4 %[v0], %[B]\n\t"
-                         "s_add_i32 m0, %[sbp], 0x400\n\t"
-                         "v_add_u32 %[v1], %[t1], %[l1]\n\t"
-                         "global_load_lds_dwordx4 %[v1], %[B]\n\t"
-                         "s_add_i32 m0, %[sbp], 0x800\n\t"
-                         "v_add_u32 %[v2], %[t2], %[l2]\n\t"
-                         "global_load_lds_dwordx4 %[v2], %[B]\n\t"
-                         "s_add_i32 m0, %[sbp], 0xc00\n\t"
-                         "v_add_u32 %[v3], %[t3], %[l3]\n\t"
-                         "global_load_lds_dwordx4 %[v3], %[B]"
-                         : [t0] "=&s"(t0), [t1] "=&s"(t1), [t2] "=&s"(t2), [t3] "=&s"(t3), [v0] "=&v"(v0),
-                           [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3)
-                         : [k0] "s"(k0), [k1] "s"(k1), [k2] "s"(k2), [k3] "s"(k3), [rb] "s"(rowbytes),
-                           [l0] "v"(voff[0]), [l1] "v"(voff[1]), [l2] "v"(voff[2]), [l3] "v"(voff[3]),
-                           [B] "s"(a.B), [sbp] "s"(sbp)
-                         : "m0", "scc");
-            if (Cfg::A_LO > 0 || pw < Cfg::A_HI) {
+            gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
+            if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
+            if (Cfg::A_LO > 0 || pw < Cfg::A_HI)
                 asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
                              "s_nop 0\n\t"
                              "global_load_lds_dwordx4 %[va], %[A]"
                              :
                              : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
                              : "m0", "scc");
-                if (Cfg::A_LO > 0 && pw < Cfg::A_HI) // a second fragment, NPROD fragments further on
-                    asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
-                                 "s_nop 0\n\t"
-                                 "global_load_lds_dwordx4 %[va], %[A]"
-                                 :
-                                 : [sbp] "s"(sbp), [arel] "s"(a_rel + NPROD * 1024), [va] "v"(va + NPROD * 1024),
-                                   [A] "s"(tileA)
-                                 : "m0", "scc");
-            }
-            va += A_FRAGS * 1024;
+            va += Cfg::A_FRAGS * 1024;
             sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
                                                                                    : sbp + STAGE_BYTES;
             issued++;
         };
 
-        // -- groups: gc* = ids of the group being issued (position 4*j + r of the producer-major
-        // copy: row r of stage j), gn* = ids of the group after it in the stream
-        auto load_group = [&](int group) __attribute__((always_inline)) {
-            return (const SHFLBW_CONST int4_t*)(kpm_all + (size_t)group * 64);
-        };
-        const SHFLBW_CONST int4_t* g = load_group(cur.y);
-        int4_t gc0 = g[0], gc1 = g[1], gc2 = g[2], gc3 = g[3];
+        // -- groups: gc* = ids of the group being issued, gn* = ids of the group after it in the
+        // stream, requested at the start of this group and first touched at its end
+        int4_t gc0 = *group_ptr(cur.y, 0), gc1 = *group_ptr(cur.y, 1), gc2 = *group_ptr(cur.y, 2),
+               gc3 = *group_ptr(cur.y, 3);
         open_tile();
+        // the ids are consumed here once, so that the loop below starts without a pending scalar
+        // load on them (it would otherwise wait, together with the loads of the following group,
+        // at the top of every iteration)
+        asm volatile("" : : "s"(gc0.x), "s"(gc1.x), "s"(gc2.x), "s"(gc3.x));
         while (true) {
-            const int ngroups = (cur.x + 3) >> 2;
+            const int nst = (cur.x + KSPS - 1) / KSPS; // stages of this tile
+            const int ngroups = (nst + NSG - 1) / NSG;
+            if (!have_next && ngroups == 1) { // the first group already needs to know what follows
+                find_next();
+                have_next = true;
+            }
             for (int q = 0; q < ngroups; q++) {
-                const int n = min(4, cur.x - 4 * q);
+                const int n = min(NSG, nst - NSG * q);
                 // the group that follows in the stream; at the very end simply this one again
                 int gnext = cur.y + q + 1;
                 if (q + 1 == ngroups) gnext = nxt.x > 0 ? nxt.y : cur.y + q;
-                const SHFLBW_CONST int4_t* gp = load_group(gnext);
-                const int4_t gn0 = gp[0], gn1 = gp[1], gn2 = gp[2], gn3 = gp[3];
-                stage(gc0.x, gc0.y, gc0.z, gc0.w);
-                if (n > 1) stage(gc1.x, gc1.y, gc1.z, gc1.w);
-                if (n > 2) stage(gc2.x, gc2.y, gc2.z, gc2.w);
-                if (n > 3) stage(gc3.x, gc3.y, gc3.z, gc3.w);
+                const int4_t gn0 = *group_ptr(gnext, 0), gn1 = *group_ptr(gnext, 1), gn2 = *group_ptr(gnext, 2),
+                             gn3 = *group_ptr(gnext, 3);
+                if (KT == 16) {
+                    stage(gc0, gc0);
+                    if (n > 1) stage(gc1, gc1);
+                    if (n > 2) stage(gc2, gc2);
+                    if (n > 3) stage(gc3, gc3);
+                } else if (RPW == 8) {
+                    stage(gc0, gc1);
+                    if (n > 1) stage(gc2, gc3);
+                } else {
+                    stage(gc0, gc0);
+                    if (n > 1) stage(gc1, gc1);
+                }
+                if (!have_next) { // deferred from the start: not needed before the first copies are out
+                    find_next();
+                    have_next = true;
+                }
                 gc0 = gn0, gc1 = gn1, gc2 = gn2, gc3 = gn3;
             }
             if (nxt.x == 0) break;
@@ -761,8 +806,9 @@ struct SpmmRsCfg {
     static constexpr int RPW = KT / NPROD;
     static constexpr int APL = A_BYTES / (NPROD * 64);    // A bytes per producer lane and stage
     static constexpr int LOADS = RPW + 1 + RPW / 4;       // vector loads per producer and stage
-    static constexpr int EPI_ROWB = WN * 2 + 16;
-    static constexpr int EPI_WAVE_BYTES = 32 * EPI_ROWB;
+    static constexpr int EPI_ROWB = 32 * 2 + 16;
+    static constexpr int EPI_ROWS = 32;
+    static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
@@ -1018,6 +1064,9 @@ static hipError_t prepare_variant()
 static const SpmmVariant g_variants[] = {
     // block 64
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
+    SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 4),
+    SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
+    SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 4),
     SHFLBW_RS_VARIANT(64, 128, 4, 4, 32, 4),
