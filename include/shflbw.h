@@ -174,6 +174,10 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  *   H, W are the INPUT extents; padding is R/2, S/2 ("same" for stride 1, as the
  *   reference's col2im, spconv/conv_format.h:77-81); Ho = (H + 2*(R/2) - R)/stride + 1.
  * Preconditions: filter synced, bcol == 1, C % 8 == 0, F % 8 == 0.
+ * init allocates device scratch inside the filter object (freed with it; states made from one
+ * filter with equal scratch size share it, so launch them on one stream); exec only launches:
+ * im2col, the SpMM kernel, and the transpose to NHWC, in order on `stream`.
+ * shflbw_spconv_init_variant: variant 0 = that pipeline, 1 = a single direct kernel.
  * ------------------------------------------------------------------------- */
 typedef struct shflbw_spconv_state {
     size_t shared_mem_size;
@@ -196,10 +200,18 @@ typedef struct shflbw_spconv_state {
     const int* packed_indices;
     const int* panel_ptr;
     int brow;
+    /* pipeline form (variant 0): im2col matrix [R*S*C][np] and filter-major result [F][np] in
+     * device scratch owned by the filter, np = B*Ho*Wo rounded up to 64; the SpMM launch state */
+    void* im2col;
+    void* result_fm;
+    int np;
+    shflbw_spmm_state spmm;
 } shflbw_spconv_state;
 
 int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* filter,
                        int B, int H, int W, int stride, const void* IFMap, void* OFMap);
+int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* filter,
+                               int B, int H, int W, int stride, const void* IFMap, void* OFMap, int variant);
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream);
 
 /* Library / device facts (for logs): compute units, clock (kHz), LDS bytes per workgroup. */

@@ -22,7 +22,7 @@ EXPORTS = [
     "shflbw_weight_sync_device", "shflbw_weight_meta_host", "shflbw_weight_device_ref",
     "shflbw_spmm_init", "shflbw_spmm_init_variant", "shflbw_spmm_exec",
     "shflbw_spmm_variant_count", "shflbw_spmm_variant_name",
-    "shflbw_spconv_init", "shflbw_spconv_exec",
+    "shflbw_spconv_init", "shflbw_spconv_init_variant", "shflbw_spconv_exec",
     "shflbw_device_info",
 ]
 
@@ -67,7 +67,8 @@ class SpconvState(C.Structure):
                 ("init_success", C.c_int), ("variant", C.c_int), ("args", _SpconvArgs),
                 ("Ho", C.c_int), ("Wo", C.c_int),
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("panel_ptr", C.c_void_p),
-                ("brow", C.c_int)]
+                ("brow", C.c_int), ("im2col", C.c_void_p), ("result_fm", C.c_void_p), ("np", C.c_int),
+                ("spmm", SpmmState)]
 
 
 _lib = None
@@ -113,6 +114,7 @@ def load():
     lib.shflbw_spmm_variant_name.restype = C.c_char_p
     lib.shflbw_spmm_variant_name.argtypes = [ci, ci]
     lib.shflbw_spconv_init.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp]
+    lib.shflbw_spconv_init_variant.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp, ci]
     lib.shflbw_spconv_exec.argtypes = [C.POINTER(SpconvState), vp]
     lib.shflbw_device_info.argtypes = [ip, ip, C.POINTER(sz), C.c_char_p, sz]
     _lib = lib

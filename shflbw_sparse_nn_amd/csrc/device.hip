@@ -31,6 +31,9 @@ void clear_device(shflbw_weight* w)
         if (*b) (void)hipFree(*b);
         *b = nullptr;
     }
+    for (auto& sc : w->conv_scratch)
+        if (sc.ptr) (void)hipFree(sc.ptr);
+    w->conv_scratch.clear();
 }
 
 static int upload_one(void** dst, const void* src, size_t bytes)
@@ -241,6 +244,12 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
 int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
                        const void* IFMap, void* OFMap)
 {
+    return shflbw_spconv_init_variant(state, f, B, H, W, stride, IFMap, OFMap, 0);
+}
+
+int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                               const void* IFMap, void* OFMap, int variant)
+{
     if (!state) return SHFLBW_ERR_INVALID;
     memset(state, 0, sizeof(*state));
     if (!f || !IFMap || !OFMap) {
@@ -277,6 +286,10 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B
         set_error("spconv_init: empty output (%d x %d)", Ho, Wo);
         return SHFLBW_ERR_SHAPE;
     }
+    if (variant != 0 && variant != 1) {
+        set_error("spconv_init: variant %d does not exist (0 = pipeline, 1 = direct kernel)", variant);
+        return SHFLBW_ERR_INVALID;
+    }
     const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
     if (!v) {
         set_error("spconv_init: no kernel for block size %d", f->brow);
@@ -307,9 +320,33 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B
     state->packed_indices = (const int*)f->d_packed_indices;
     state->panel_ptr = (const int*)f->d_group_ptr;
     state->brow = f->brow;
-    state->variant = 0;
+    state->variant = variant;
     state->shared_mem_size = (size_t)v->lds_bytes;
     const long npix = (long)B * Ho * Wo;
+    if (variant == 0) {
+        // pipeline form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
+        const long np = (npix + 63) / 64 * 64;
+        const long K = (long)f->R * f->S * f->C;
+        if (np > 0x7fffffffL || (unsigned long long)K * (unsigned long long)np * 2ull > 0xffffffffull) {
+            set_error("spconv_init: problem too large for the pipeline form (im2col matrix of %ld x %ld)", K, np);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        const size_t bm_bytes = (size_t)K * np * 2, dm_bytes = (size_t)f->F * np * 2;
+        const size_t bytes = bm_bytes + dm_bytes;
+        shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is not part of the weight's value
+        void* scratch = nullptr;
+        for (auto& sc : fw->conv_scratch)
+            if (sc.bytes == bytes) scratch = sc.ptr;
+        if (!scratch) {
+            SHFLBW_HIP_TRY(hipMalloc(&scratch, bytes));
+            fw->conv_scratch.push_back({bytes, scratch});
+        }
+        state->im2col = scratch;
+        state->result_fm = (char*)scratch + bm_bytes;
+        state->np = (int)np;
+        int rc = shflbw_spmm_init(&state->spmm, f, (int)np, state->im2col, nullptr, state->result_fm, 1.f, 0.f);
+        if (rc != SHFLBW_OK) return rc;
+    }
     state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
     state->grid_dim[1] = state->grid_dim[2] = 1;
     state->block_dim[0] = (unsigned)v->threads;
@@ -347,6 +384,22 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
+    if (state->variant == 0) {
+        hipError_t e = launch_im2col_nhwc(a, (half_t*)state->im2col, state->np, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: im2col launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        int rc = shflbw_spmm_exec(&state->spmm, stream);
+        if (rc != SHFLBW_OK) return rc;
+        e = launch_transpose_to_nhwc((const half_t*)state->result_fm, a.out, a.F, a.B * a.Ho * a.Wo, state->np,
+                                     (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: transpose launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        return SHFLBW_OK;
+    }
     hipError_t e = v->launch(a, (hipStream_t)stream);
     if (e != hipSuccess) {
         set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));

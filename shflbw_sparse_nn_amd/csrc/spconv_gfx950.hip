@@ -156,6 +156,104 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
     }
 }
 
+
+// =======================================================================================
+// Pipeline form of the convolution (the default): three launches on the caller's stream
+//   1. im2col_nhwc_kernel:   NHWC input -> im2col matrix Bm[k][p], k = (r,s,c), p = output pixel,
+//                            rows of NP fp16 (NP = pixel count rounded up to 64), zero outside the image
+//   2. the SpMM kernel:      Dm[f][p] = A_sparse * Bm (row permutation applied to f)
+//   3. transpose_to_nhwc_kernel: Dm[f][p] -> OFMap[p][f]
+// The gather that the sparse filter needs is a gather of whole rows of a [k][pixel] matrix; NHWC
+// keeps channels, not pixels, contiguous, and a row-permuted filter scatters its output channels,
+// so both ends are turned into plain 64 x 64 tile transposes and the middle is the tuned SpMM.
+// =======================================================================================
+constexpr int TT = 64;            // transpose tile edge
+constexpr int TT_LD = TT + 8;     // LDS row length in halves (16-byte aligned rows, spread over banks)
+
+// 256 threads move a 64 x 64 fp16 tile: `load(i, j)` returns the 16-byte piece j (8 halves) of source
+// row i; `store(o, q, v)` receives the 8 halves at source rows 8q .. 8q+7 of source column o.
+template <typename Load, typename Store>
+__device__ __forceinline__ void transpose_tile_64(half_t (*tile)[TT_LD], Load load, Store store)
+{
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        const int i = (t >> 3) + pass * 32, j = t & 7;
+        *(half8_t*)&tile[i][j * 8] = load(i, j);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        const int o = (t >> 3) + pass * 32, q = t & 7;
+        half8_t v;
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][o];
+        store(o, q, v);
+    }
+}
+
+// grid: (pixel tiles, channel tiles, taps); block 256
+__global__ void __launch_bounds__(256) im2col_nhwc_kernel(const half_t* __restrict__ in, half_t* __restrict__ bm, int B,
+                                                          int H, int W, int C, int S, int stride, int pad_h, int pad_w,
+                                                          int Ho, int Wo, int NP)
+{
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT_LD];
+    const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT;
+    const int r = blockIdx.z / S, s = blockIdx.z - r * S;
+    const int npix = B * Ho * Wo;
+    transpose_tile_64(
+        tile,
+        [&](int i, int j) { // source row = output pixel p0 + i, piece = channels c0 + 8j ..
+            const int p = p0 + i, c = c0 + j * 8;
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (p < npix && c < C) {
+                const int wo = p % Wo, ho = (p / Wo) % Ho, b = p / (Wo * Ho);
+                const int hi = ho * stride - pad_h + r, wi = wo * stride - pad_w + s;
+                if (hi >= 0 && hi < H && wi >= 0 && wi < W)
+                    v = *(const half8_t*)(in + ((size_t)(b * H + hi) * W + wi) * C + c);
+            }
+            return v;
+        },
+        [&](int o, int q, half8_t v) { // destination row k = tap * C + c0 + o, pixels p0 + 8q ..
+            const int c = c0 + o;
+            if (c < C) *(half8_t*)(bm + ((size_t)blockIdx.z * C + c) * NP + p0 + q * 8) = v;
+        });
+}
+
+// grid: (pixel tiles, filter tiles); block 256
+__global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __restrict__ dm, half_t* __restrict__ out,
+                                                                int F, int npix, int NP)
+{
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT_LD];
+    const int p0 = blockIdx.x * TT, f0 = blockIdx.y * TT;
+    transpose_tile_64(
+        tile,
+        [&](int i, int j) { // source row = filter f0 + i, piece = pixels p0 + 8j ..
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (f0 + i < F) v = *(const half8_t*)(dm + (size_t)(f0 + i) * NP + p0 + j * 8);
+            return v;
+        },
+        [&](int o, int q, half8_t v) { // destination row = pixel p0 + o, filters f0 + 8q ..
+            const int pix = p0 + o, f = f0 + q * 8;
+            if (pix < npix && f < F) *(half8_t*)(out + (size_t)pix * F + f) = v;
+        });
+}
+
+hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream)
+{
+    const dim3 grid(NP / TT, (a.C + TT - 1) / TT, a.R * a.S);
+    hipLaunchKernelGGL(im2col_nhwc_kernel, grid, dim3(256), 0, stream, a.in, bm, a.B, a.H, a.W, a.C, a.S, a.stride,
+                       a.pad_h, a.pad_w, a.Ho, a.Wo, NP);
+    return hipGetLastError();
+}
+
+hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int npix, int NP, hipStream_t stream)
+{
+    const dim3 grid(NP / TT, (F + TT - 1) / TT);
+    hipLaunchKernelGGL(transpose_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, npix, NP);
+    return hipGetLastError();
+}
+
 template <int V, int WN, int NWAVES, int KT>
 static hipError_t launch_conv(const SpconvLaunchArgs& a, hipStream_t stream)
 {

@@ -29,4 +29,9 @@ struct SpconvVariant {
 
 const SpconvVariant* spconv_variants(int* count);
 
+// Stages 1 and 3 of the pipeline form of the convolution: NHWC input -> im2col matrix with rows of NP
+// halves (NP a multiple of 64), and filter-major result -> NHWC output.
+hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream);
+hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int npix, int NP, hipStream_t stream);
+
 } // namespace shflbw

@@ -39,6 +39,15 @@ struct shflbw_weight {
     void* d_packed_indices = nullptr;
     void* d_packed_indices_pm = nullptr;
     void* d_packed_values = nullptr;
+
+    // device scratch of the pipeline form of the convolution (im2col matrix followed by the
+    // filter-major result), one allocation per distinct size, handed out by shflbw_spconv_init
+    // and kept until the weight is re-initialised or destroyed
+    struct Scratch {
+        size_t bytes;
+        void* ptr;
+    };
+    std::vector<Scratch> conv_scratch;
 };
 
 namespace shflbw {

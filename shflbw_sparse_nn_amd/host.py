@@ -172,14 +172,17 @@ class SpmmBlockwiseOp:
 
 
 class SpconvBlockwiseOp:
-    """initialize(spfilter, B, H, W, stride, IFMap, OFMap); NHWC tensors, H and W are input extents."""
+    """initialize(spfilter, B, H, W, stride, IFMap, OFMap); NHWC tensors, H and W are input extents.
+    variant 0 (default): im2col + SpMM + transpose on the stream; variant 1: one direct kernel."""
 
-    def __init__(self):
+    def __init__(self, variant=0):
         self._lib = capi.load()
         self._state = capi.SpconvState()
+        self._variant = variant
 
     def initialize(self, spfilter, B, H, W, stride, IFMap, OFMap):
-        capi.check(self._lib.shflbw_spconv_init(C.byref(self._state), spfilter._h, B, H, W, stride, IFMap, OFMap))
+        capi.check(self._lib.shflbw_spconv_init_variant(C.byref(self._state), spfilter._h, B, H, W, stride, IFMap,
+                                                        OFMap, self._variant))
         self._keep = spfilter
         return self._state
 

@@ -39,11 +39,11 @@ def run_spmm(torch, w, B, Cmat=None, alpha=1.0, beta=None, variant=-1, poison=Tr
     return dD.cpu().numpy()
 
 
-def run_spconv(torch, w, R, Sx, Cc, x_nhwc, stride):
+def run_spconv(torch, w, R, Sx, Cc, x_nhwc, stride, variant=0):
     f = upload_weight(w, R, Sx, Cc, cls=S.BlockwiseSpFilter)
     Bn, H, W, _ = x_nhwc.shape
     dX = to_dev(torch, x_nhwc)
-    op = S.SpconvBlockwiseOp()
+    op = S.SpconvBlockwiseOp(variant)
     Ho = (H + 2 * (R // 2) - R) // stride + 1
     Wo = (W + 2 * (Sx // 2) - Sx) // stride + 1
     dY = torch.full((Bn, Ho, Wo, w["nrow"]), float("nan"), dtype=torch.float16, device="cuda")

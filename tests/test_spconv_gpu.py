@@ -19,10 +19,11 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    got = run_spconv(torch, w, R, S, C, x, stride)
-    assert got.shape == ref.shape
-    assert not np.isnan(got.astype(np.float32)).any(), "kernel left output elements unwritten"
-    np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16))
+    for variant in (0, 1):  # 0: im2col + SpMM + transpose (default), 1: one direct kernel
+        got = run_spconv(torch, w, R, S, C, x, stride, variant)
+        assert got.shape == ref.shape
+        assert not np.isnan(got.astype(np.float32)).any(), "variant %d left output elements unwritten" % variant
+        np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16), err_msg="variant %d" % variant)
 
 
 @pytest.mark.parametrize("Bn,H,W,C,F,R,S,stride,V,d,permute", [
