@@ -36,7 +36,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=11)
-    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (cfg1 is the graded headline)")
+    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D)")
     ap.add_argument("--variant", type=int, default=-1, help="force a tile variant (default: library choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--traffic", default=None,
@@ -56,6 +56,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.config in P.CONV_CONFIGS:
+        return bench_conv(args, np, torch, S, P)
     c = P.SPMM_CONFIGS[args.config]
     M, K, N, V, d = c["M"], c["K"], c["N"], c["V"], c["d"]
     w = P.make_weight(M, K, V, d, True, 2021, dist=c["a_dist"])
@@ -203,6 +205,82 @@ def main():
         "device": S.device_info(),
     }
     print(json.dumps(out))
+
+
+def bench_conv(args, np, torch, S, P):
+    """Secondary workloads: the sparse Conv2D configs (cfg3, cfg4), NHWC, one step = one exec of the
+    operator (im2col, SpMM and transpose launches on one stream).  Same JSON shape as the headline."""
+    from oracle import oracle as O
+    from tests.gpu_util import to_dev, upload_weight
+    c = P.CONV_CONFIGS[args.config]
+    B, H, W, C, F, R, Sx, stride, V, d = [c[k] for k in ("B", "H", "W", "C", "F", "R", "S", "stride", "V", "d")]
+    Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
+    npix = B * Ho * Wo
+    stream = torch.cuda.current_stream()
+
+    def make_op(w, x):
+        f = upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
+        dX = to_dev(torch, x)
+        dY = torch.full((B, Ho, Wo, F), float("nan"), dtype=torch.float16, device="cuda")
+        op = S.SpconvBlockwiseOp(max(args.variant, 0))
+        op.initialize(f, B, H, W, stride, dX.data_ptr(), dY.data_ptr())
+        return op, f, dX, dY
+
+    # correctness gate: bit-exact against the oracle on the integer twin
+    wi = P.make_weight(F, R * Sx * C, V, d, True, 2021, integer=True)
+    xi = np.random.default_rng(2022).integers(-4, 5, size=(B, H, W, C)).astype(np.float16)
+    opi, fi, dXi, dYi = make_op(wi, xi)
+    opi(stream.cuda_stream)
+    torch.cuda.synchronize()
+    ref_i = O.float_to_half(P.conv_oracle(wi, R, Sx, C, xi, stride))
+    if not np.array_equal(dYi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
+        print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
+        sys.exit(1)
+    del opi, fi, dXi, dYi
+
+    w = P.make_weight(F, R * Sx * C, V, d, True, 2021, dist=c["w_dist"])
+    x = P.make_dense(B * H * W, C, 2021, dist=c["x_dist"]).reshape(B, H, W, C)
+    op, f, dX, dY = make_op(w, x)
+    nnzb = w["nnzb"]
+    eff_flops = 2.0 * nnzb * V * npix
+    alg_bytes = nnzb * V * 2 + (nnzb + F // V + 1 + F) * 4 + B * H * W * C * 2 + npix * F * 2
+    for _ in range(args.warmup):
+        op(stream.cuda_stream)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(args.steps):
+        op(stream.cuda_stream)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    t = ms * 1e-3
+    cpu = None
+    if not args.no_cpu:
+        t0 = time.time()
+        P.conv_oracle(w, R, Sx, C, x, stride)
+        t_all = time.time() - t0
+        cpu = {"value": round(eff_flops / t_all / 1e12, 6), "unit": "TFLOP/s", "cores": O.max_threads(), "kind": "port",
+               "sample": "whole workload, one pass: %.2f s" % t_all}
+    ai = eff_flops / alg_bytes
+    mfma_bound = ai * HBM_PEAK_GBS * 1e9 > MFMA_F16_PEAK_TFLOPS * 1e12
+    eff_tflops = eff_flops / t / 1e12
+    roof = ({"bound": "mfma", "achieved": round(eff_tflops, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": round(eff_tflops / MFMA_F16_PEAK_TFLOPS, 4)} if mfma_bound else
+            {"bound": "hbm", "achieved": round(alg_bytes / t / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(alg_bytes / t / 1e9 / HBM_PEAK_GBS, 4)})
+    roof.update({"traffic": None, "algorithmic_bytes": alg_bytes, "effective_flops": eff_flops})
+    print(json.dumps({
+        "metric": "effective sparse TFLOP/s + %% fp16 MFMA peak, SpConv2D %s" % args.config,
+        "value": round(eff_tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter N(0, 0.05), input N(0, 1)",
+        "config": {"workload": "%s: sparse Conv2D NHWC %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
+                               "nnzb=%d" % (args.config, B, H, W, C, F, R, Sx, stride, V, d, nnzb),
+                   "kernel": "pipeline: im2col + SpMM + transpose" if args.variant <= 0 else "direct"},
+        "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
+        "roofline": roof, "cpu_baseline": cpu, "device": S.device_info()}))
 
 
 if __name__ == "__main__":

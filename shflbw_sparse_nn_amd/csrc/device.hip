@@ -361,7 +361,7 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         set_error("spconv_exec: state was not initialised successfully");
         return SHFLBW_ERR_STATE;
     }
-    const SpconvVariant* v = find_spconv_variant(state->brow, state->variant, nullptr);
+    const SpconvVariant* v = find_spconv_variant(state->brow, 0, nullptr); // the direct kernel of this block size
     if (!v) return SHFLBW_ERR_UNSUPPORTED;
     SpconvLaunchArgs a;
     a.B = state->args.B;

@@ -167,27 +167,29 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
 // keeps channels, not pixels, contiguous, and a row-permuted filter scatters its output channels,
 // so both ends are turned into plain 64 x 64 tile transposes and the middle is the tuned SpMM.
 // =======================================================================================
-constexpr int TT = 64;            // transpose tile edge
-constexpr int TT_LD = TT + 8;     // LDS row length in halves (16-byte aligned rows, spread over banks)
+constexpr int TT = 64; // transpose tile edge
 
 // 256 threads move a 64 x 64 fp16 tile: `load(i, j)` returns the 16-byte piece j (8 halves) of source
 // row i; `store(o, q, v)` receives the 8 halves at source rows 8q .. 8q+7 of source column o.
+// Piece j of row i sits at piece position j ^ (i / 8) of its LDS row, so the eight row groups a
+// wave reads in one instruction fall into eight different bank groups.
 template <typename Load, typename Store>
-__device__ __forceinline__ void transpose_tile_64(half_t (*tile)[TT_LD], Load load, Store store)
+__device__ __forceinline__ void transpose_tile_64(half_t (*tile)[TT], Load load, Store store)
 {
     const int t = threadIdx.x;
 #pragma unroll
     for (int pass = 0; pass < 2; pass++) {
         const int i = (t >> 3) + pass * 32, j = t & 7;
-        *(half8_t*)&tile[i][j * 8] = load(i, j);
+        *(half8_t*)&tile[i][(j ^ ((i >> 3) & 7)) * 8] = load(i, j);
     }
     __syncthreads();
 #pragma unroll
     for (int pass = 0; pass < 2; pass++) {
         const int o = (t >> 3) + pass * 32, q = t & 7;
+        const int c = (((o >> 3) ^ q) << 3) | (o & 7);
         half8_t v;
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][o];
+        for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][c];
         store(o, q, v);
     }
 }
@@ -197,7 +199,7 @@ __global__ void __launch_bounds__(256) im2col_nhwc_kernel(const half_t* __restri
                                                           int H, int W, int C, int S, int stride, int pad_h, int pad_w,
                                                           int Ho, int Wo, int NP)
 {
-    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT_LD];
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
     const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT;
     const int r = blockIdx.z / S, s = blockIdx.z - r * S;
     const int npix = B * Ho * Wo;
@@ -224,7 +226,7 @@ __global__ void __launch_bounds__(256) im2col_nhwc_kernel(const half_t* __restri
 __global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __restrict__ dm, half_t* __restrict__ out,
                                                                 int F, int npix, int NP)
 {
-    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT_LD];
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
     const int p0 = blockIdx.x * TT, f0 = blockIdx.y * TT;
     transpose_tile_64(
         tile,
