@@ -194,32 +194,61 @@ __device__ __forceinline__ void transpose_tile_64(half_t (*tile)[TT], Load load,
     }
 }
 
-// grid: (pixel tiles, channel tiles, taps); block 256
+// grid: (pixel tiles, channel tiles, filter rows r); block 256.  A workgroup walks the S taps of its
+// filter row: the pixel decode is done once, and the loads of the next tap are in flight while the
+// current one goes through LDS.
 __global__ void __launch_bounds__(256) im2col_nhwc_kernel(const half_t* __restrict__ in, half_t* __restrict__ bm, int B,
                                                           int H, int W, int C, int S, int stride, int pad_h, int pad_w,
                                                           int Ho, int Wo, int NP)
 {
     __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
-    const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT;
-    const int r = blockIdx.z / S, s = blockIdx.z - r * S;
+    const int t = threadIdx.x;
+    const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT, r = blockIdx.z;
     const int npix = B * Ho * Wo;
-    transpose_tile_64(
-        tile,
-        [&](int i, int j) { // source row = output pixel p0 + i, piece = channels c0 + 8j ..
-            const int p = p0 + i, c = c0 + j * 8;
-            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (p < npix && c < C) {
-                const int wo = p % Wo, ho = (p / Wo) % Ho, b = p / (Wo * Ho);
-                const int hi = ho * stride - pad_h + r, wi = wo * stride - pad_w + s;
-                if (hi >= 0 && hi < H && wi >= 0 && wi < W)
-                    v = *(const half8_t*)(in + ((size_t)(b * H + hi) * W + wi) * C + c);
-            }
-            return v;
-        },
-        [&](int o, int q, half8_t v) { // destination row k = tap * C + c0 + o, pixels p0 + 8q ..
-            const int c = c0 + o;
-            if (c < C) *(half8_t*)(bm + ((size_t)blockIdx.z * C + c) * NP + p0 + q * 8) = v;
-        });
+    // the two source pieces of this thread: pixels p0 + i, channels c0 + 8j ..
+    const int j = t & 7, c = c0 + j * 8;
+    long base[2]; // element offset of (b, hi, wi = wo*stride - pad_w, c)
+    bool row_ok[2]; // the input row hi exists
+    int wi0[2];
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        const int p = p0 + (t >> 3) + pass * 32;
+        const int wo = p % Wo, ho = (p / Wo) % Ho, b = p / (Wo * Ho);
+        const int hi = ho * stride - pad_h + r;
+        wi0[pass] = wo * stride - pad_w;
+        row_ok[pass] = p < npix && c < C && hi >= 0 && hi < H;
+        base[pass] = ((long)(b * H + hi) * W + wi0[pass]) * C + c;
+    }
+    auto fetch = [&](int s, int pass) {
+        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int wi = wi0[pass] + s;
+        if (row_ok[pass] && wi >= 0 && wi < W) v = *(const half8_t*)(in + base[pass] + (long)s * C);
+        return v;
+    };
+    half8_t nxt[2] = {fetch(0, 0), fetch(0, 1)};
+    for (int s = 0; s < S; s++) {
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++) {
+            const int i = (t >> 3) + pass * 32;
+            *(half8_t*)&tile[i][(j ^ ((i >> 3) & 7)) * 8] = nxt[pass];
+        }
+        __syncthreads();
+        if (s + 1 < S) {
+            nxt[0] = fetch(s + 1, 0);
+            nxt[1] = fetch(s + 1, 1);
+        }
+        const int tap = r * S + s;
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++) {
+            const int o = (t >> 3) + pass * 32, q = t & 7;
+            const int col = (((o >> 3) ^ q) << 3) | (o & 7);
+            half8_t v;
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][col];
+            if (c0 + o < C) *(half8_t*)(bm + ((size_t)tap * C + c0 + o) * NP + p0 + q * 8) = v;
+        }
+        __syncthreads();
+    }
 }
 
 // grid: (pixel tiles, filter tiles); block 256
@@ -243,7 +272,7 @@ __global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __
 
 hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream)
 {
-    const dim3 grid(NP / TT, (a.C + TT - 1) / TT, a.R * a.S);
+    const dim3 grid(NP / TT, (a.C + TT - 1) / TT, a.R);
     hipLaunchKernelGGL(im2col_nhwc_kernel, grid, dim3(256), 0, stream, a.in, bm, a.B, a.H, a.W, a.C, a.S, a.stride,
                        a.pad_h, a.pad_w, a.Ho, a.Wo, NP);
     return hipGetLastError();
