@@ -290,12 +290,14 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         set_error("spconv_init: variant %d does not exist (0 = pipeline, 1 = direct kernel)", variant);
         return SHFLBW_ERR_INVALID;
     }
-    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
-    if (!v) {
-        set_error("spconv_init: no kernel for block size %d", f->brow);
-        return SHFLBW_ERR_UNSUPPORTED;
+    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
+    if (variant == 1) {
+        if (!v) {
+            set_error("spconv_init: no direct kernel for block size %d", f->brow);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        SHFLBW_HIP_TRY(v->prepare());
     }
-    SHFLBW_HIP_TRY(v->prepare());
     shflbw_device_ref ref;
     shflbw_weight_device_ref(f, &ref);
     state->args.B = B;
@@ -321,7 +323,6 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     state->panel_ptr = (const int*)f->d_group_ptr;
     state->brow = f->brow;
     state->variant = variant;
-    state->shared_mem_size = (size_t)v->lds_bytes;
     const long npix = (long)B * Ho * Wo;
     if (variant == 0) {
         // pipeline form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
@@ -347,9 +348,16 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         int rc = shflbw_spmm_init(&state->spmm, f, (int)np, state->im2col, nullptr, state->result_fm, 1.f, 0.f);
         if (rc != SHFLBW_OK) return rc;
     }
-    state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
+    if (variant == 1) {
+        state->shared_mem_size = (size_t)v->lds_bytes;
+        state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
+        state->block_dim[0] = (unsigned)v->threads;
+    } else { // the figures of the middle (SpMM) launch
+        state->shared_mem_size = state->spmm.shared_mem_size;
+        state->grid_dim[0] = state->spmm.grid_dim[0];
+        state->block_dim[0] = state->spmm.block_dim[0];
+    }
     state->grid_dim[1] = state->grid_dim[2] = 1;
-    state->block_dim[0] = (unsigned)v->threads;
     state->block_dim[1] = state->block_dim[2] = 1;
     state->init_success = 1;
     return SHFLBW_OK;
@@ -362,7 +370,7 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         return SHFLBW_ERR_STATE;
     }
     const SpconvVariant* v = find_spconv_variant(state->brow, 0, nullptr); // the direct kernel of this block size
-    if (!v) return SHFLBW_ERR_UNSUPPORTED;
+    if (!v && state->variant == 1) return SHFLBW_ERR_UNSUPPORTED;
     SpconvLaunchArgs a;
     a.B = state->args.B;
     a.H = state->args.H;

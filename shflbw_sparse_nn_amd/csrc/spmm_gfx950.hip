@@ -273,15 +273,18 @@ __device__ __forceinline__ int ks_sel(const int (&ks)[N_], int base, int sub, in
 // fragment sets) so that its LDS reads really run one stage ahead of the MFMAs.
 // Tiles are dealt so that the workgroups of one XCD work on the same B column slab.
 // =======================================================================================
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER_ = false>
 struct SpmmWsCfg {
+    static constexpr bool DEFER = DEFER_;                 // stores of a tile trickle out during the next tile
     static constexpr int BN = WN * NCONS;
     static constexpr int MB = V / 32;
     static constexpr int NB = WN / 32;
     static constexpr int ROWB = BN * 2;
     static constexpr int B_BYTES = KT * ROWB;
-    static constexpr int KSPS = KT / 16;                  // MFMA k-steps per stage
-    static constexpr int A_FRAGS = KSPS * MB;             // 1 KiB fragments per stage, contiguous in memory and LDS
+    static constexpr int KSPS = KT / 16;                  // 16-slot steps per stage
+    // 1 KiB A fragments per stage, contiguous in memory and LDS: V >= 32 has V/32 per 16-slot step
+    // (32x32x16 tiles), V == 16 has one per 32-slot step (16x16x32 tiles)
+    static constexpr int A_FRAGS = V == 16 ? KT / 32 : KSPS * MB;
     static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
     static constexpr int RPW = KT / NPROD;                // gathered rows (= copies) per producer and stage
     static constexpr int A_HI = A_FRAGS % NPROD;          // producers [0, A_HI) copy one more A fragment
@@ -289,11 +292,12 @@ struct SpmmWsCfg {
     static constexpr int OPS = RPW + A_LO;                // copies per stage every producer issues at least
     static constexpr int EPI_ROWB = 32 * 2 + 16;
     static constexpr int EPI_ROWS = NCONS > 4 ? 16 : 32;  // rows of a 32 x 32 accumulator block staged at a time
-    static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
+    static constexpr int DST_ROWB = WN * 2 + 16;          // DEFER: a consumer's whole fp16 sub-tile, row + 16 bytes
+    static constexpr int EPI_WAVE_BYTES = DEFER ? V * DST_ROWB : EPI_ROWS * EPI_ROWB;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
-    static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
+    static_assert((V % 32 == 0 || (V == 16 && KT == 32 && !DEFER)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
     static_assert(BN == 512, "one gathered row is exactly one 1 KiB copy instruction");
     static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
     static_assert(A_LO <= 1 && (A_LO == 0 || A_HI == 0), "at most one A fragment per producer and stage");
@@ -384,6 +388,35 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
         }
     };
 
+    // DEFER: the finished tile is parked as fp16 in this wave's LDS area (row r at r * DST_ROWB, its
+    // output row index in the 16 bytes behind the row) and leaves in 1 KiB steps, one per stage of
+    // the following tile, so that the stores of all compute units do not hit memory in one burst
+    // while the matrix cores wait.
+    constexpr int DRAIN_ROWS = 1024 / (WN * 2);          // rows per step (a wave stores 64 x 16 bytes)
+    constexpr int DRAIN_STEPS = V / DRAIN_ROWS;
+    constexpr int DPR = WN / 8;                          // 16-byte pieces per row
+    const uint32_t dhome = epi + (lane / DPR) * Cfg::DST_ROWB + (lane % DPR) * 16;
+    uint32_t dpos = dhome; // this lane's piece of the next step
+    int pending = 0;       // steps still parked
+    int dcol = 0;          // column of the lane's piece in D (of the parked tile)
+    auto drain_step = [&]() __attribute__((always_inline)) {
+        if (pending > 0) {
+            half8_t v = *(SHFLBW_LDS half8_t*)(uintptr_t)dpos;
+            const int orow = *(SHFLBW_LDS int*)(uintptr_t)(dpos - (lane % DPR) * 16 + WN * 2);
+            if (dcol < N) {
+                const size_t off = (size_t)orow * N + dcol;
+                if (a.beta != 0.f) {
+                    const half8_t c = *(const half8_t*)(a.C + off);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] = (half_t)((float)v[e] + a.beta * (float)c[e]);
+                }
+                *(half8_t*)(a.D + off) = v;
+            }
+            dpos += DRAIN_ROWS * Cfg::DST_ROWB;
+            pending--;
+        }
+    };
+
     TileWalker w;
     w.init(a.panel_desc, id_first, id_end, S, X);
     bool primed = false; // fragments of the upcoming stage are in f0
@@ -431,6 +464,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             __builtin_amdgcn_sched_barrier(0);
             mma(cur);
             __builtin_amdgcn_sched_barrier(0);
+            if (Cfg::DEFER) drain_step();
         };
 
         if (ntl > 0 && !primed) { // very first stage of the stream
@@ -461,6 +495,32 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             }
         }
 
+        if (Cfg::DEFER) {
+            while (pending > 0) drain_step(); // a short tile did not give the parked one enough steps
+            const uint32_t wr = epi + (lane & 31) * Cfg::DST_ROWB + (lane >> 5) * 8;
+            const bool scale = alpha != 1.f;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                    for (int ig = 0; ig < 4; ig++) {
+                        half4_t h;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            h[e] = (half_t)(scale ? acc[mb][nb][ig * 4 + e] * alpha : acc[mb][nb][ig * 4 + e]);
+                        *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + mb * 32 * Cfg::DST_ROWB + nb * 64 + ig * 16) = h;
+                    }
+            // lane l of register q holds the output row of stored row 64 q + l
+#pragma unroll
+            for (int q = 0; q < (V + 63) / 64; q++)
+                if (q * 64 + lane < V)
+                    *(SHFLBW_LDS int*)(uintptr_t)(epi + (q * 64 + lane) * Cfg::DST_ROWB + WN * 2) = rid[q];
+            dpos = dhome;
+            dcol = n0 + cw * WN + (lane % DPR) * 8;
+            pending = DRAIN_STEPS;
+            continue;
+        }
         // ---- epilogue of this wave's V x WN sub-tile, one 32 x 32 accumulator block at a time:
         // fp16 (one rounding) -> private LDS area (a lane holds 4 consecutive columns of one row
         // per 8-byte write) -> 16-byte pieces of 64-byte row segments -> scattered rows of D.  The
@@ -539,6 +599,126 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             for (int mb = 0; mb < MB; mb++) epi_block(mb, T{}, T{});
         }
     }
+    if (Cfg::DEFER)
+        while (pending > 0) drain_step();
+}
+
+// Consumer role for block height 16: 16x16x32 tiles, one 32-slot step per LDS stage, same barrier
+// protocol and ring as ws_consumer.  Wave `cw` owns the 16 x WN sub-tile at column cw*WN.  A lane of
+// the result holds output row lane % 16 and, per 16-column block, the 4 columns 4*(lane/16) + 0..3.
+template <typename Cfg, int WN, int NCONS>
+__device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
+                                              int id_end, int S)
+{
+    constexpr int V = 16, BN = Cfg::BN, NB = WN / 16, ROWB = Cfg::ROWB;
+    constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
+    static_assert(Cfg::KSPS == 2 && WN % 64 == 0, "one 32-slot step per stage");
+    const int N = a.N, X = a.X;
+    const int li = lane & 15;
+    uint32_t boff[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        const int unit = (cw * WN + nb * 16) / 16;
+        boff[nb] = (uint32_t)((8 * (lane >> 4) + (li >> 2)) * ROWB + ((unit ^ row_xor32(li >> 2)) << 5) + ((li & 3) << 3));
+    }
+    const uint32_t aoff = (uint32_t)(B_BYTES + lane * 16);
+    const uint32_t epi = lds0 + Cfg::RING_BYTES + cw * Cfg::EPI_WAVE_BYTES;
+
+    struct Frags {
+        half8_t a, b[NB];
+    };
+    Frags f0, f1;
+    auto load_frags = [&](uint32_t sbase, Frags& f) __attribute__((always_inline)) {
+        f.a = *(SHFLBW_LDS half8_t*)(uintptr_t)(sbase + aoff);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const half4_t lo = lds_read_tr16(sbase + boff[nb]);
+            const half4_t hi = lds_read_tr16(sbase + boff[nb] + 4 * ROWB);
+            f.b[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+
+    TileWalker w;
+    w.init(a.panel_desc, id_first, id_end, S, X);
+    bool primed = false;
+    uint32_t sb = lds0;
+    const float alpha = a.alpha, beta = a.beta;
+    for (; w.valid(); w.advance()) {
+        const int panel = w.id % X;
+        const int n0 = (w.id / X) * BN;
+        const int ntl = (w.cur.x + 1) >> 1; // 32-slot steps
+
+        float4_t acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const int srow = panel * V + li;
+        const int orow = a.row_ids ? a.row_ids[srow] : srow;
+
+        auto mma = [&](const Frags& f) __attribute__((always_inline)) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.b[nb], f.a, acc[nb], 0, 0, 0);
+        };
+        auto stage = [&](Frags& cur, Frags& nxt) __attribute__((always_inline)) {
+            sb = (sb + STAGE_BYTES == lds0 + Cfg::RING_BYTES) ? lds0 : sb + STAGE_BYTES;
+            wg_barrier();
+            load_frags(sb, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(cur);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if (ntl > 0 && !primed) {
+            wg_barrier();
+            load_frags(sb, f0);
+            primed = true;
+        }
+        int s = 0;
+        for (; s + 1 < ntl; s += 2) {
+            stage(f0, f1);
+            stage(f1, f0);
+        }
+        if (s < ntl) {
+            stage(f0, f1);
+            f0 = f1;
+        }
+
+        // ---- epilogue: 16 rows x 64 columns at a time through the private LDS area (row of 128
+        // bytes + 16), read back as 16-byte pieces of 128-byte row segments, 8 rows per store
+        constexpr int EROWB = 64 * 2 + 16;
+        static_assert(16 * EROWB <= Cfg::EPI_WAVE_BYTES, "epilogue staging area");
+        const uint32_t wr = epi + li * EROWB + (lane >> 4) * 8;
+        const uint32_t rd = epi + (lane >> 3) * EROWB + (lane & 7) * 16;
+        size_t roff[2];
+#pragma unroll
+        for (int it = 0; it < 2; it++) roff[it] = (size_t)__shfl(orow, it * 8 + (lane >> 3)) * N;
+#pragma unroll
+        for (int h = 0; h < WN / 64; h++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                half4_t hv;
+#pragma unroll
+                for (int e = 0; e < 4; e++) hv[e] = (half_t)(acc[h * 4 + q][e] * alpha);
+                *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + q * 32) = hv;
+            }
+            half8_t v[2];
+#pragma unroll
+            for (int it = 0; it < 2; it++) v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * 8 * EROWB);
+            const int col = n0 + cw * WN + h * 64 + (lane & 7) * 8;
+            if (col < N) {
+                if (beta != 0.f) {
+                    half8_t c[2];
+#pragma unroll
+                    for (int it = 0; it < 2; it++) c[it] = *(const half8_t*)(a.C + roff[it] + col);
+#pragma unroll
+                    for (int it = 0; it < 2; it++)
+#pragma unroll
+                        for (int e = 0; e < 8; e++) v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
+                }
+#pragma unroll
+                for (int it = 0; it < 2; it++) *(half8_t*)(a.D + roff[it] + col) = v[it];
+            }
+        }
+    }
 }
 
 // Four gathered rows of B (ids k, wave-uniform) into four consecutive 1 KiB LDS rows starting
@@ -575,10 +755,10 @@ __device__ __forceinline__ void gather_rows4(int4_t k, uint32_t rowbytes, const 
                  : "m0", "scc");
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
 __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
     constexpr int BN = Cfg::BN, RPW = Cfg::RPW;
     constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
 
@@ -747,13 +927,16 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         return;
     }
 
-    ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
+    if constexpr (V == 16)
+        ws_consumer16<Cfg, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
+    else
+        ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
 static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
     SpmmLaunchArgs b = a;
     b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
     const int T = a.X * b.n_tiles;
@@ -764,16 +947,16 @@ static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
     grid = (grid / 8) * 8;
     const int need = ((T + 7) / 8) * 8;
     if (grid > need) grid = need;
-    hipLaunchKernelGGL((spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid), dim3(Cfg::THREADS),
-                       Cfg::LDS_BYTES, stream, b);
+    hipLaunchKernelGGL((spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>), dim3(grid),
+                       dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, b);
     return hipGetLastError();
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
 static hipError_t prepare_ws()
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
-    return hipFuncSetAttribute((const void*)spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
+    return hipFuncSetAttribute((const void*)spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
 }
 
@@ -808,6 +991,8 @@ struct SpmmRsCfg {
     static constexpr int LOADS = RPW + 1 + RPW / 4;       // vector loads per producer and stage
     static constexpr int EPI_ROWB = 32 * 2 + 16;
     static constexpr int EPI_ROWS = 32;
+    static constexpr bool DEFER = false;
+    static constexpr int DST_ROWB = WN * 2 + 16;
     static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
@@ -1025,6 +1210,13 @@ static hipError_t prepare_rs()
             &prepare_rs<V, WN, NC, NP, KT, D>                                                                 \
     }
 
+#define SHFLBW_WSD_VARIANT(V, WN, NC, NP, KT, NS)                                                            \
+    {                                                                                                        \
+        V, WN* NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS, true>::LDS_BYTES,                         \
+            "wsd" #V "x" #WN "x" #NC "c" #NP "p_k" #KT "_s" #NS, &launch_ws<V, WN, NC, NP, KT, NS, true>,    \
+            &prepare_ws<V, WN, NC, NP, KT, NS, true>                                                          \
+    }
+
 #define SHFLBW_WS_VARIANT(V, WN, NC, NP, KT, NS)                                                             \
     {                                                                                                        \
         V, WN* NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS>::LDS_BYTES,                               \
@@ -1064,6 +1256,7 @@ static hipError_t prepare_variant()
 static const SpmmVariant g_variants[] = {
     // block 64
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
+    SHFLBW_WSD_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
@@ -1086,6 +1279,8 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
     SHFLBW_VARIANT(32, 64, 2, 32, 3),
+    // block 16
+    SHFLBW_WS_VARIANT(16, 128, 4, 4, 32, 4),
     // block 128
     SHFLBW_VARIANT(128, 64, 4, 32, 3),
     SHFLBW_VARIANT(128, 32, 4, 32, 3),

@@ -29,7 +29,7 @@ def _exact_case(torch, M, N, K, V, d, permute, variant=-1, seed=2021):
 
 
 # the reference's own test case: N = 960 exercises the column-residue path
-@pytest.mark.parametrize("V", [32, 64, 128])
+@pytest.mark.parametrize("V", [16, 32, 64, 128])
 @pytest.mark.parametrize("permute", [False, True])
 def test_reference_case_all_variants(torch_gpu, V, permute):
     for variant in range(len(S.spmm_variants(V))):
@@ -44,6 +44,8 @@ def test_reference_case_all_variants(torch_gpu, V, permute):
     (256, 128, 1024, 128, 0.3),
     (512, 1032, 777, 32, 0.2),  # K not a multiple of anything
     (1024, 1024, 1024, 64, 0.25),  # cfg0 shape
+    (48, 72, 40, 16, 0.7),      # block height 16: three panels, ragged N and K
+    (512, 1000, 513, 16, 0.15),
 ])
 def test_exact_shapes(torch_gpu, M, N, K, V, d):
     _exact_case(torch_gpu, M, N, K, V, d, True)
@@ -74,10 +76,11 @@ def test_empty_panels_write_zeros(torch_gpu):
     assert X == 4 and (got[np.sort(w["row_permute_ids"][:V])] == 0).all()
 
 
+@pytest.mark.parametrize("V", [16, 32])
 @pytest.mark.parametrize("permute", [False, True])
-def test_beta_c_epilogue(torch_gpu, permute):
+def test_beta_c_epilogue(torch_gpu, permute, V):
     # D = A*B + C, the overload the reference's example uses (example/spmm.blockwise.cu:50)
-    M, N, K, V = 256, 256, 256, 32
+    M, N, K = 256, 256, 256
     w = P.make_weight(M, K, V, 0.2, permute, 11, integer=True)
     B = P.make_dense(K, N, 11, integer=True)
     Cm = P.make_dense(M, N, 11, integer=True, stream=3)
