@@ -273,9 +273,8 @@ __device__ __forceinline__ int ks_sel(const int (&ks)[N_], int base, int sub, in
 // fragment sets) so that its LDS reads really run one stage ahead of the MFMAs.
 // Tiles are dealt so that the workgroups of one XCD work on the same B column slab.
 // =======================================================================================
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER_ = false>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 struct SpmmWsCfg {
-    static constexpr bool DEFER = DEFER_;                 // stores of a tile trickle out during the next tile
     static constexpr int BN = WN * NCONS;
     static constexpr int MB = V / 32;
     static constexpr int NB = WN / 32;
@@ -292,18 +291,21 @@ struct SpmmWsCfg {
     static constexpr int OPS = RPW + A_LO;                // copies per stage every producer issues at least
     static constexpr int EPI_ROWB = 32 * 2 + 16;
     static constexpr int EPI_ROWS = NCONS > 4 ? 16 : 32;  // rows of a 32 x 32 accumulator block staged at a time
-    static constexpr int DST_ROWB = WN * 2 + 16;          // DEFER: a consumer's whole fp16 sub-tile, row + 16 bytes
-    static constexpr int EPI_WAVE_BYTES = DEFER ? V * DST_ROWB : EPI_ROWS * EPI_ROWB;
+    static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
-    static_assert((V % 32 == 0 || (V == 16 && KT == 32 && !DEFER)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
+    static_assert((V % 32 == 0 || (V == 16 && KT == 32)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
     static_assert(BN == 512, "one gathered row is exactly one 1 KiB copy instruction");
     static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
     static_assert(A_LO <= 1 && (A_LO == 0 || A_HI == 0), "at most one A fragment per producer and stage");
+    // A producer passes one barrier before every stage it issues.  The barrier in front of stage j is the
+    // one after which the consumers no longer read stage j - NSTAGE, i.e. their barrier number j - (NSTAGE-2):
+    // the consumers therefore pass NSTAGE - 2 extra barriers before their first one.
+    static constexpr int START_BARRIERS = NSTAGE - 2;
     static_assert(THREADS <= 1024, "workgroup size limit");
     static_assert(NSTAGE >= 3, "one stage computed, one landed, one in flight");
-    static_assert((NSTAGE - 3) * OPS < 64, "vmcnt is a 6-bit counter");
+    static_assert((NSTAGE - 3) * (RPW + 1) < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 };
 
@@ -311,6 +313,18 @@ __device__ __forceinline__ void wg_barrier()
 {
     // bare barrier: no implied wait on outstanding global stores or copies
     asm volatile("s_barrier" ::: "memory");
+}
+
+// The NSTAGE - 1 barriers a producer passes after its last stage: number U of them waits until at most
+// NSTAGE - 3 - U stages of OPS copies each are outstanding.
+template <int U, int NSTAGE, int OPS>
+__device__ __forceinline__ void producer_tail()
+{
+    if constexpr (U < NSTAGE - 1) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3 - U > 0 ? NSTAGE - 3 - U : 0) * OPS));
+        wg_barrier();
+        producer_tail<U + 1, NSTAGE, OPS>();
+    }
 }
 
 // Walks the tile ids id, id+S, ... < end of one workgroup and keeps the descriptor of the
@@ -348,9 +362,9 @@ struct TileWalker {
 
 // Consumer role of the role-split kernels: wave `cw` of NCONS owns the V x WN sub-tile at column
 // cw*WN of every tile of the workgroup.  `Cfg` describes the LDS ring (stage size and count) and the
-// per-wave epilogue area; the barrier protocol is: barrier number t (counted from 0) is passed once
-// stage t of the workgroup's stage stream is complete in LDS; a consumer executes one barrier before
-// its first stage and one more per stage.
+// per-wave epilogue area; the barrier protocol is: after START_BARRIERS start-up barriers, barrier
+// number t (counted from 0) is passed once stage t of the workgroup's stage stream is complete in
+// LDS; a consumer executes one barrier before its first stage and one more per stage.
 template <typename Cfg, int V, int WN, int NCONS>
 __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
                                             int id_end, int S)
@@ -385,35 +399,6 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             const half4_t lo = lds_read_tr16(sbase + boff[nb]);
             const half4_t hi = lds_read_tr16(sbase + boff[nb] + 4 * ROWB);
             f.b[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-    };
-
-    // DEFER: the finished tile is parked as fp16 in this wave's LDS area (row r at r * DST_ROWB, its
-    // output row index in the 16 bytes behind the row) and leaves in 1 KiB steps, one per stage of
-    // the following tile, so that the stores of all compute units do not hit memory in one burst
-    // while the matrix cores wait.
-    constexpr int DRAIN_ROWS = 1024 / (WN * 2);          // rows per step (a wave stores 64 x 16 bytes)
-    constexpr int DRAIN_STEPS = V / DRAIN_ROWS;
-    constexpr int DPR = WN / 8;                          // 16-byte pieces per row
-    const uint32_t dhome = epi + (lane / DPR) * Cfg::DST_ROWB + (lane % DPR) * 16;
-    uint32_t dpos = dhome; // this lane's piece of the next step
-    int pending = 0;       // steps still parked
-    int dcol = 0;          // column of the lane's piece in D (of the parked tile)
-    auto drain_step = [&]() __attribute__((always_inline)) {
-        if (pending > 0) {
-            half8_t v = *(SHFLBW_LDS half8_t*)(uintptr_t)dpos;
-            const int orow = *(SHFLBW_LDS int*)(uintptr_t)(dpos - (lane % DPR) * 16 + WN * 2);
-            if (dcol < N) {
-                const size_t off = (size_t)orow * N + dcol;
-                if (a.beta != 0.f) {
-                    const half8_t c = *(const half8_t*)(a.C + off);
-#pragma unroll
-                    for (int e = 0; e < 8; e++) v[e] = (half_t)((float)v[e] + a.beta * (float)c[e]);
-                }
-                *(half8_t*)(a.D + off) = v;
-            }
-            dpos += DRAIN_ROWS * Cfg::DST_ROWB;
-            pending--;
         }
     };
 
@@ -455,19 +440,31 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
         // (that stage has landed once the barrier is passed; past the end of the stream the reads
         // hit a stale slot and are never used).  Padded k-steps have zero A values, so every step
         // is computed unconditionally and the loop body stays branch-free.
+        // Scheduling pattern for "load_frags(next); mma(current)": the MFMAs only need registers that
+        // were filled a stage ago, so they start right away and the LDS reads are spread behind them,
+        // RPM reads per MFMA; the remaining MFMAs follow the last read.
+        auto interleave_reads = [&]() __attribute__((always_inline)) {
+            constexpr int NRD = MB + 2 * NB, NMM = MB * NB, RPM = (NRD + NMM - 1) / NMM, G = (NRD + RPM - 1) / RPM;
+            static_assert(G <= NMM, "every group of reads sits behind an MFMA");
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0); // LDS reads
+            }
+            if (NMM - G > 0) __builtin_amdgcn_sched_group_barrier(0x008, NMM - G, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
         auto stage = [&](Frags& cur, Frags& nxt) __attribute__((always_inline)) {
             sb = (sb + STAGE_BYTES == lds0 + Cfg::RING_BYTES) ? lds0 : sb + STAGE_BYTES;
             wg_barrier();
-            // scheduling fences: the reads of the following fragments must be issued before the
-            // MFMAs that overlap them, not sunk down to their first use
             load_frags(sb, 0, nxt);
-            __builtin_amdgcn_sched_barrier(0);
             mma(cur);
-            __builtin_amdgcn_sched_barrier(0);
-            if (Cfg::DEFER) drain_step();
+            interleave_reads();
         };
 
         if (ntl > 0 && !primed) { // very first stage of the stream
+#pragma unroll
+            for (int i = 0; i < Cfg::START_BARRIERS; i++) wg_barrier();
             wg_barrier();
             load_frags(sb, 0, f0);
             primed = true;
@@ -488,39 +485,12 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             // number of steps computes one padded step (zero A values).
             for (int p = 0; p < (ntl + 1) >> 1; p++) {
                 load_frags(sb, 1, f1);
-                __builtin_amdgcn_sched_barrier(0);
                 mma(f0);
-                __builtin_amdgcn_sched_barrier(0);
+                interleave_reads();
                 stage(f1, f0);
             }
         }
 
-        if (Cfg::DEFER) {
-            while (pending > 0) drain_step(); // a short tile did not give the parked one enough steps
-            const uint32_t wr = epi + (lane & 31) * Cfg::DST_ROWB + (lane >> 5) * 8;
-            const bool scale = alpha != 1.f;
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-                    for (int ig = 0; ig < 4; ig++) {
-                        half4_t h;
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            h[e] = (half_t)(scale ? acc[mb][nb][ig * 4 + e] * alpha : acc[mb][nb][ig * 4 + e]);
-                        *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + mb * 32 * Cfg::DST_ROWB + nb * 64 + ig * 16) = h;
-                    }
-            // lane l of register q holds the output row of stored row 64 q + l
-#pragma unroll
-            for (int q = 0; q < (V + 63) / 64; q++)
-                if (q * 64 + lane < V)
-                    *(SHFLBW_LDS int*)(uintptr_t)(epi + (q * 64 + lane) * Cfg::DST_ROWB + WN * 2) = rid[q];
-            dpos = dhome;
-            dcol = n0 + cw * WN + (lane % DPR) * 8;
-            pending = DRAIN_STEPS;
-            continue;
-        }
         // ---- epilogue of this wave's V x WN sub-tile, one 32 x 32 accumulator block at a time:
         // fp16 (one rounding) -> private LDS area (a lane holds 4 consecutive columns of one row
         // per 8-byte write) -> 16-byte pieces of 64-byte row segments -> scattered rows of D.  The
@@ -599,8 +569,6 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
             for (int mb = 0; mb < MB; mb++) epi_block(mb, T{}, T{});
         }
     }
-    if (Cfg::DEFER)
-        while (pending > 0) drain_step();
 }
 
 // Consumer role for block height 16: 16x16x32 tiles, one 32-slot step per LDS stage, same barrier
@@ -668,6 +636,8 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
             __builtin_amdgcn_sched_barrier(0);
         };
         if (ntl > 0 && !primed) {
+#pragma unroll
+            for (int i = 0; i < Cfg::START_BARRIERS; i++) wg_barrier();
             wg_barrier();
             load_frags(sb, f0);
             primed = true;
@@ -755,10 +725,10 @@ __device__ __forceinline__ void gather_rows4(int4_t k, uint32_t rowbytes, const 
                  : "m0", "scc");
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
     constexpr int BN = Cfg::BN, RPW = Cfg::RPW;
     constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES;
 
@@ -791,7 +761,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         const int pw = wave - NCONS;
         const uint32_t rowbytes = (uint32_t)N * 2;
         const SHFLBW_CONST int2_t* desc = (const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc;
-        constexpr int OPS = Cfg::OPS, KSPS = Cfg::KSPS;
+        constexpr int KSPS = Cfg::KSPS;
         constexpr int NSG = 64 / KT; // stages per group
         // ids of a group for this producer, as int4 number q.  Four rows per producer and stage:
         // stage j uses int4 j - with 16-row stages from the producer-major copy [16 pw + 4 j + r],
@@ -838,92 +808,100 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             }
         };
 
-        // -- ring position of the next stage: LDS address of this wave's rows
-        uint32_t sbp = lds0 + pw * RPW * 1024;
-        const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's A fragment slot relative to sbp
-        int issued = 0;
-        // one stage: optional wait + barrier, then the copies
-        auto stage = [&](int4_t ka, int4_t kb) __attribute__((always_inline)) {
-            if (issued >= NSTAGE - 2) {
-                // barrier g = issued - (NSTAGE-1): stage g+1 must have landed, NSTAGE-3 younger
-                // stages may stay in flight
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * OPS));
+        // -- everything on the stage cadence, specialised on whether this producer also copies an A
+        // fragment per stage: its copies per stage are then a compile-time number and the waits exact
+        auto run = [&](auto has_a_tag) __attribute__((always_inline)) {
+            constexpr bool HAS_A = decltype(has_a_tag)::value;
+            constexpr int MYOPS = RPW + (HAS_A ? 1 : 0); // copies per stage of this producer
+            // ring position of the next stage: LDS address of this wave's rows
+            uint32_t sbp = lds0 + pw * RPW * 1024;
+            const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's A fragment slot relative to sbp
+            // One stage, branch-free: the barrier in front of stage j tells that the consumers are done with
+            // the ring slot it overwrites; before arriving there the stage the consumers read next (issued
+            // NSTAGE - 2 stages ago) must have landed, NSTAGE - 3 younger stages stay in flight.  In front
+            // of the first stages nothing is outstanding and the wait falls through.
+            auto stage = [&](int4_t ka, int4_t kb) __attribute__((always_inline)) {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * MYOPS));
                 wg_barrier();
-            }
-            gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
-            if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
-            if (Cfg::A_LO > 0 || pw < Cfg::A_HI)
-                asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
-                             "s_nop 0\n\t"
-                             "global_load_lds_dwordx4 %[va], %[A]"
-                             :
-                             : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
-                             : "m0", "scc");
-            va += Cfg::A_FRAGS * 1024;
-            sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
-                                                                                   : sbp + STAGE_BYTES;
-            issued++;
-        };
+                gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
+                if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
+                if (HAS_A)
+                    asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
+                                 "s_nop 0\n\t"
+                                 "global_load_lds_dwordx4 %[va], %[A]"
+                                 :
+                                 : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
+                                 : "m0", "scc");
+                va += Cfg::A_FRAGS * 1024;
+                sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
+                                                                                       : sbp + STAGE_BYTES;
+            };
 
-        // -- groups: gc* = ids of the group being issued, gn* = ids of the group after it in the
-        // stream, requested at the start of this group and first touched at its end
-        int4_t gc0 = *group_ptr(cur.y, 0), gc1 = *group_ptr(cur.y, 1), gc2 = *group_ptr(cur.y, 2),
-               gc3 = *group_ptr(cur.y, 3);
-        open_tile();
-        // the ids are consumed here once, so that the loop below starts without a pending scalar
-        // load on them (it would otherwise wait, together with the loads of the following group,
-        // at the top of every iteration)
-        asm volatile("" : : "s"(gc0.x), "s"(gc1.x), "s"(gc2.x), "s"(gc3.x));
-        while (true) {
-            const int nst = (cur.x + KSPS - 1) / KSPS; // stages of this tile
-            const int ngroups = (nst + NSG - 1) / NSG;
-            if (!have_next && ngroups == 1) { // the first group already needs to know what follows
-                find_next();
-                have_next = true;
-            }
-            for (int q = 0; q < ngroups; q++) {
-                const int n = min(NSG, nst - NSG * q);
-                // the group that follows in the stream; at the very end simply this one again
-                int gnext = cur.y + q + 1;
-                if (q + 1 == ngroups) gnext = nxt.x > 0 ? nxt.y : cur.y + q;
-                const int4_t gn0 = *group_ptr(gnext, 0), gn1 = *group_ptr(gnext, 1), gn2 = *group_ptr(gnext, 2),
-                             gn3 = *group_ptr(gnext, 3);
-                if (KT == 16) {
-                    stage(gc0, gc0);
-                    if (n > 1) stage(gc1, gc1);
-                    if (n > 2) stage(gc2, gc2);
-                    if (n > 3) stage(gc3, gc3);
-                } else if (RPW == 8) {
-                    stage(gc0, gc1);
-                    if (n > 1) stage(gc2, gc3);
-                } else {
-                    stage(gc0, gc0);
-                    if (n > 1) stage(gc1, gc1);
-                }
-                if (!have_next) { // deferred from the start: not needed before the first copies are out
+            // -- groups: gc* = ids of the group being issued, gn* = ids of the group after it in the
+            // stream, requested at the start of this group and first touched at its end
+            int4_t gc0 = *group_ptr(cur.y, 0), gc1 = *group_ptr(cur.y, 1), gc2 = *group_ptr(cur.y, 2),
+                   gc3 = *group_ptr(cur.y, 3);
+            open_tile();
+            // the ids are consumed here once, so that the loop below starts without a pending scalar
+            // load on them (it would otherwise wait, together with the loads of the following group,
+            // at the top of every iteration)
+            asm volatile("" : : "s"(gc0.x), "s"(gc1.x), "s"(gc2.x), "s"(gc3.x));
+            while (true) {
+                const int nst = (cur.x + KSPS - 1) / KSPS; // stages of this tile
+                const int ngroups = (nst + NSG - 1) / NSG;
+                if (!have_next && ngroups == 1) { // the first group already needs to know what follows
                     find_next();
                     have_next = true;
                 }
-                gc0 = gn0, gc1 = gn1, gc2 = gn2, gc3 = gn3;
+                for (int q = 0; q < ngroups; q++) {
+                    const int n = min(NSG, nst - NSG * q);
+                    // the group that follows in the stream; at the very end simply this one again
+                    int gnext = cur.y + q + 1;
+                    if (q + 1 == ngroups) gnext = nxt.x > 0 ? nxt.y : cur.y + q;
+                    const int4_t gn0 = *group_ptr(gnext, 0), gn1 = *group_ptr(gnext, 1), gn2 = *group_ptr(gnext, 2),
+                                 gn3 = *group_ptr(gnext, 3);
+                    if (n == NSG) { // whole group: straight-line code
+                        if (KT == 16) {
+                            stage(gc0, gc0);
+                            stage(gc1, gc1);
+                            stage(gc2, gc2);
+                            stage(gc3, gc3);
+                        } else if (RPW == 8) {
+                            stage(gc0, gc1);
+                            stage(gc2, gc3);
+                        } else {
+                            stage(gc0, gc0);
+                            stage(gc1, gc1);
+                        }
+                    } else if (KT == 16) { // last, partial group of a tile
+                        stage(gc0, gc0);
+                        if (n > 1) stage(gc1, gc1);
+                        if (n > 2) stage(gc2, gc2);
+                    } else if (RPW == 8) {
+                        stage(gc0, gc1);
+                    } else {
+                        stage(gc0, gc0);
+                    }
+                    if (!have_next) { // deferred from the start: not needed before the first copies are out
+                        find_next();
+                        have_next = true;
+                    }
+                    gc0 = gn0, gc1 = gn1, gc2 = gn2, gc3 = gn3;
+                }
+                if (nxt.x == 0) break;
+                id = idn, cur = nxt;
+                find_next();
+                open_tile();
             }
-            if (nxt.x == 0) break;
-            id = idn, cur = nxt;
-            find_next();
-            open_tile();
-        }
-        // -- tail: `issued` stages are out, barriers g = issued-(NSTAGE-1) ... issued-1 remain
-        for (int g2 = max(issued - (NSTAGE - 1), -1); g2 < issued; g2++) {
-            const int younger = issued - g2 - 2; // stages issued after stage g2+1, which must have landed
-            if (NSTAGE > 5 && younger >= 3)
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * OPS));
-            else if (NSTAGE > 4 && younger == 2)
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * OPS));
-            else if (NSTAGE > 3 && younger == 1)
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(1 * OPS));
-            else
-                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            wg_barrier();
-        }
+            // -- tail: the consumers pass NSTAGE - 1 more barriers.  Barrier number u of them stands in front
+            // of the stage issued NSTAGE - 2 - u stages ago (NSTAGE - 3 - u younger ones may be in flight);
+            // the last one only releases the consumers' final stage.
+            producer_tail<0, NSTAGE, MYOPS>();
+        };
+        if (Cfg::A_LO > 0 || pw < Cfg::A_HI)
+            run(std::true_type{});
+        else
+            run(std::false_type{});
         return;
     }
 
@@ -933,10 +911,10 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
     SpmmLaunchArgs b = a;
     b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
     const int T = a.X * b.n_tiles;
@@ -947,275 +925,18 @@ static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
     grid = (grid / 8) * 8;
     const int need = ((T + 7) / 8) * 8;
     if (grid > need) grid = need;
-    hipLaunchKernelGGL((spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>), dim3(grid),
+    hipLaunchKernelGGL((spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid),
                        dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, b);
     return hipGetLastError();
 }
 
-template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE, bool DEFER = false>
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
 static hipError_t prepare_ws()
 {
-    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>;
-    return hipFuncSetAttribute((const void*)spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE, DEFER>,
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    return hipFuncSetAttribute((const void*)spmm_shflbw_ws_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
 }
-
-// =======================================================================================
-// Register-staged variant of the role-split kernel.
-//
-// The gather has a latency of one to two microseconds (part of every stage misses the L2), so
-// keeping the matrix cores fed needs on the order of ten stages in flight per compute unit -
-// more bytes than the LDS can hold.  Here the producers therefore gather with ordinary vector
-// loads into a ring of registers DEPTH stages deep (a producer wave has 64 KiB of registers and
-// nothing else to keep in them) and move a stage into a short LDS ring only when it has
-// arrived.  All loads are visible to the compiler, which counts the in-order vector-memory
-// counter exactly; the kept-column ids ride the same counter (one 16-byte uniform load per
-// stage and producer, fetched a further DEPTH stages ahead).
-// LDS ring: stage t lives in slot t % 3.  A consumer has finished reading stage t when it
-// arrives at barrier t+2, the producers write stage t after barrier t-1: three slots suffice.
-// =======================================================================================
-template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
-struct SpmmRsCfg {
-    static constexpr int NSTAGE = 3;
-    static constexpr int KSPS = KT / 16;                  // MFMA k-steps per LDS stage
-    static constexpr int BN = WN * NCONS;
-    static constexpr int MB = V / 32;
-    static constexpr int NB = WN / 32;
-    static constexpr int ROWB = BN * 2;
-    static constexpr int B_BYTES = KT * ROWB;
-    static constexpr int A_FRAGS = MB;                    // per k-step
-    static constexpr int A_BYTES = KSPS * A_FRAGS * 1024; // per stage, contiguous in memory and in LDS
-    static constexpr int STAGE_BYTES = B_BYTES + A_BYTES;
-    static constexpr int RPW = KT / NPROD;
-    static constexpr int APL = A_BYTES / (NPROD * 64);    // A bytes per producer lane and stage
-    static constexpr int LOADS = RPW + 1 + RPW / 4;       // vector loads per producer and stage
-    static constexpr int EPI_ROWB = 32 * 2 + 16;
-    static constexpr int EPI_ROWS = 32;
-    static constexpr bool DEFER = false;
-    static constexpr int DST_ROWB = WN * 2 + 16;
-    static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
-    static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
-    static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
-    static constexpr int THREADS = (NCONS + NPROD) * 64;
-    static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
-    static_assert(BN == 512, "one gathered row is one 1 KiB wave access");
-    static_assert((KT == 16 || KT == 32) && NPROD == 4, "four producers, one or two k16 steps per stage");
-    static_assert(APL == 4 || APL == 8 || APL == 16, "the A block of a stage splits evenly over the producer lanes");
-    static_assert(DEPTH * LOADS < 64, "vmcnt is a 6-bit counter");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
-};
-
-// Cursor over the stages of a workgroup's non-empty tiles, in stream order.  Past the last stage
-// it stays on the last stage (`done` set), so that addresses derived from it remain valid: the
-// producers' pipeline issues a fixed number of loads per step and simply re-reads that stage.
-struct StageCursor {
-    int id, idn, end, S, X; // current tile, next non-empty tile, range end, stride, panels
-    int2_t cur, nxt;        // descriptors {k16 steps, first 64-slot group}; cur.x == 0: no stage at all
-    int ti;                 // stage inside the current tile
-    int kshift;             // log2 of the k16 steps per stage
-    bool done;
-    __device__ __forceinline__ int stages() const { return (cur.x + (1 << kshift) - 1) >> kshift; }
-    const SHFLBW_CONST int2_t* desc;
-    __device__ __forceinline__ void find_next()
-    {
-        nxt.x = 0;
-        for (idn += S; idn < end; idn += S) {
-            nxt = desc[idn % X];
-            if (nxt.x > 0) break;
-        }
-    }
-    __device__ __forceinline__ void init(const int* d, int first, int end_, int S_, int X_, int kshift_)
-    {
-        desc = (const SHFLBW_CONST int2_t*)(uintptr_t)d;
-        end = end_, S = S_, X = X_, ti = 0, kshift = kshift_;
-        idn = first - S;
-        nxt.x = 0, nxt.y = 0;
-        find_next();
-        id = idn, cur = nxt;
-        done = cur.x == 0;
-        if (!done) find_next();
-    }
-    // returns true when the step entered a new tile
-    __device__ __forceinline__ bool advance()
-    {
-        if (ti + 1 < stages()) {
-            ti++;
-            return false;
-        }
-        if (nxt.x == 0) {
-            done = true;
-            return false;
-        }
-        ti = 0, id = idn, cur = nxt;
-        find_next();
-        return true;
-    }
-};
-
-template <int BYTES> struct LaneChunk;
-template <> struct LaneChunk<4> { typedef int type; };
-template <> struct LaneChunk<8> { typedef int2_t type; };
-template <> struct LaneChunk<16> { typedef int4_t type; };
-
-template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
-__global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_rs_kernel(SpmmLaunchArgs a)
-{
-    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
-    constexpr int BN = Cfg::BN, RPW = Cfg::RPW, APL = Cfg::APL;
-    constexpr int STAGE_BYTES = Cfg::STAGE_BYTES, B_BYTES = Cfg::B_BYTES, A_BYTES = Cfg::A_BYTES;
-    // the A block of a stage is moved in equal shares by all producers, so every producer issues
-    // exactly the same loads per stage
-    typedef typename LaneChunk<APL>::type achunk_t;
-
-    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int N = a.N, X = a.X;
-
-    // same tile -> workgroup map as the copy-based kernel: XCD x owns a contiguous id range
-    const int T = X * a.n_tiles;
-    const int per = (T + 7) >> 3;
-    const int xcd = blockIdx.x & 7;
-    const int S = gridDim.x >> 3;
-    const int id_first = xcd * per + (blockIdx.x >> 3);
-    const int id_end = min(T, (xcd + 1) * per);
-
-    if (wave < NCONS) {
-        ws_consumer<Cfg, V, WN, NCONS>(a, lds0, lane, wave, id_first, id_end, S);
-        return;
-    }
-
-    // =========================== producer ===========================
-    // Everything on the stage cadence is unconditional: the compiler derives exact vmcnt waits only
-    // when every path through the loop issues the same loads in the same order.
-    const int pw = wave - NCONS;
-    // a zero the compiler cannot see through: added to wave-uniform addresses so that the id loads
-    // stay vector loads (a scalar load would need a full wait and has no place in this pipeline)
-    uint32_t vzero = 0;
-    asm volatile("" : "+v"(vzero));
-
-    StageCursor ic, rc; // the id-load cursor runs DEPTH stages ahead of the row-load cursor
-    ic.init(a.panel_desc, id_first, id_end, S, X, Cfg::KSPS == 2 ? 1 : 0);
-    if (ic.done) return; // no stage: the consumers execute no barrier either
-    rc = ic;
-
-    half8_t rb[DEPTH][RPW]; // gathered rows in flight
-    achunk_t ra[DEPTH];     // A shares in flight
-    int4_t ri[DEPTH][RPW / 4]; // ids of the stage whose rows are requested next from this ring position
-
-    auto load_ids = [&](int4_t (&dst)[RPW / 4]) __attribute__((always_inline)) {
-        const int* p = a.kidx + ((size_t)ic.cur.y * 64 + ic.ti * KT + pw * RPW);
-#pragma unroll
-        for (int q = 0; q < RPW / 4; q++) dst[q] = *(const int4_t*)((const char*)p + q * 16 + vzero);
-        ic.advance();
-    };
-
-    // per-tile state of the row cursor
-    uint32_t voff[4];                                     // lane byte offsets inside a B row, by row % 4
-    const uint32_t aoff = pw * (64 * APL) + lane * APL;   // lane byte offset inside the A block of a stage
-    const char* tileA = nullptr;                          // A blocks of the current tile
-    auto open_tile = [&]() __attribute__((always_inline)) {
-        const int n0 = (rc.id / X) * BN;
-        tileA = (const char*)a.packedA + (size_t)rc.cur.y * (64 * V * 2);
-#pragma unroll
-        for (int j = 0; j < 4; j++) { // RPW is a multiple of 4: row pw*RPW + j has swizzle key j % 4
-            const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
-            const int col = n0 + lc * 8;
-            voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
-        }
-    };
-    const size_t rowbytes = (size_t)N * 2;
-    int real = 0; // stages of the stream whose rows have been requested
-    auto load_rows = [&](const int4_t (&ids)[RPW / 4], half8_t (&dstb)[RPW], achunk_t& dsta) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            const int k = __builtin_amdgcn_readfirstlane(ids[r / 4][r % 4]);
-            dstb[r] = *(const half8_t*)((const char*)a.B + (size_t)(uint32_t)k * rowbytes + voff[r & 3]);
-        }
-        dsta = *(const achunk_t*)(tileA + (size_t)rc.ti * A_BYTES + aoff);
-        if (!rc.done) {
-            real++;
-            if (rc.advance()) open_tile();
-        }
-    };
-
-    // ---- prologue: ids of the first DEPTH stages, their rows, and the ids of the DEPTH after them
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) load_ids(ri[j]);
-    open_tile();
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) {
-        load_rows(ri[j], rb[j], ra[j]);
-        load_ids(ri[j]);
-    }
-
-    // ---- stage t: move it from the registers into LDS slot t % 3, request stage t + DEPTH into the
-    // same registers, pass barrier t
-    const uint32_t wr_b = lds0 + pw * RPW * 1024 + lane * 16;
-    const uint32_t wr_a = lds0 + B_BYTES + aoff;
-    uint32_t slot = 0; // byte offset of the LDS slot of the stage moved next
-    auto move_stage = [&](half8_t (&srcb)[RPW], achunk_t& srca, int4_t (&ids)[RPW / 4]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < RPW; r++) *(SHFLBW_LDS half8_t*)(uintptr_t)(wr_b + slot + r * 1024) = srcb[r];
-        *(SHFLBW_LDS achunk_t*)(uintptr_t)(wr_a + slot) = srca;
-        slot = (slot + STAGE_BYTES == Cfg::RING_BYTES) ? 0 : slot + STAGE_BYTES;
-        load_rows(ids, srcb, srca);
-        load_ids(ids);
-        __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the LDS writes of this stage are done
-        wg_barrier();
-    };
-    int t = 0;
-    // steady state: DEPTH real stages are resident in the ring
-    while (real - t >= DEPTH) {
-#pragma unroll
-        for (int j = 0; j < DEPTH; j++) move_stage(rb[j], ra[j], ri[j]);
-        t += DEPTH;
-    }
-    // tail of the stream: fewer than DEPTH stages left, ring positions 0 .. real - t - 1
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++)
-        if (t + j < real) move_stage(rb[j], ra[j], ri[j]);
-    wg_barrier(); // the consumers' last stage passes one more barrier
-}
-
-template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
-static hipError_t launch_rs(const SpmmLaunchArgs& a, hipStream_t stream)
-{
-    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
-    SpmmLaunchArgs b = a;
-    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
-    const int T = a.X * b.n_tiles;
-    int grid = a.num_cus > 0 ? a.num_cus : 256;
-    grid = (grid / 8) * 8;
-    const int need = ((T + 7) / 8) * 8;
-    if (grid > need) grid = need;
-    hipLaunchKernelGGL((spmm_shflbw_rs_kernel<V, WN, NCONS, NPROD, KT, DEPTH>), dim3(grid), dim3(Cfg::THREADS),
-                       Cfg::LDS_BYTES, stream, b);
-    return hipGetLastError();
-}
-
-template <int V, int WN, int NCONS, int NPROD, int KT, int DEPTH>
-static hipError_t prepare_rs()
-{
-    using Cfg = SpmmRsCfg<V, WN, NCONS, NPROD, KT, DEPTH>;
-    return hipFuncSetAttribute((const void*)spmm_shflbw_rs_kernel<V, WN, NCONS, NPROD, KT, DEPTH>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-}
-
-#define SHFLBW_RS_VARIANT(V, WN, NC, NP, KT, D)                                                              \
-    {                                                                                                        \
-        V, WN* NC, (NC + NP) * 64, SpmmRsCfg<V, WN, NC, NP, KT, D>::LDS_BYTES,                                \
-            "rs" #V "x" #WN "x" #NC "c" #NP "p_k" #KT "_d" #D, &launch_rs<V, WN, NC, NP, KT, D>,             \
-            &prepare_rs<V, WN, NC, NP, KT, D>                                                                 \
-    }
-
-#define SHFLBW_WSD_VARIANT(V, WN, NC, NP, KT, NS)                                                            \
-    {                                                                                                        \
-        V, WN* NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS, true>::LDS_BYTES,                         \
-            "wsd" #V "x" #WN "x" #NC "c" #NP "p_k" #KT "_s" #NS, &launch_ws<V, WN, NC, NP, KT, NS, true>,    \
-            &prepare_ws<V, WN, NC, NP, KT, NS, true>                                                          \
-    }
 
 #define SHFLBW_WS_VARIANT(V, WN, NC, NP, KT, NS)                                                             \
     {                                                                                                        \
@@ -1256,16 +977,11 @@ static hipError_t prepare_variant()
 static const SpmmVariant g_variants[] = {
     // block 64
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
-    SHFLBW_WSD_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 4),
-    SHFLBW_RS_VARIANT(64, 128, 4, 4, 32, 4),
-    SHFLBW_RS_VARIANT(64, 128, 4, 4, 32, 3),
-    SHFLBW_RS_VARIANT(64, 128, 4, 4, 16, 8),
-    SHFLBW_RS_VARIANT(64, 128, 4, 4, 16, 4),
     SHFLBW_VARIANT(64, 64, 4, 32, 3),
     SHFLBW_VARIANT(64, 64, 4, 32, 2),
     SHFLBW_VARIANT(64, 64, 4, 16, 4),
