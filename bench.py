@@ -278,7 +278,8 @@ def bench_conv(args, np, torch, S, P):
         "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter N(0, 0.05), input N(0, 1)",
         "config": {"workload": "%s: sparse Conv2D NHWC %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
                                "nnzb=%d" % (args.config, B, H, W, C, F, R, Sx, stride, V, d, nnzb),
-                   "kernel": "pipeline: im2col + SpMM + transpose" if args.variant <= 0 else "direct"},
+                   "kernel": {0: "plane layout + SpMM (tap offsets in the gather) + transpose", 1: "direct",
+                              2: "im2col matrix + SpMM + transpose"}[max(args.variant, 0)]},
         "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
         "roofline": roof, "cpu_baseline": cpu, "device": S.device_info()}))
 

@@ -151,6 +151,7 @@ typedef struct shflbw_spmm_state {
     const int* packed_indices_pm;
     const int* panel_ptr;
     int brow;
+    int ldb_bytes; /* distance in bytes between two rows of B that are one kept-column id apart: N * 2 */
 } shflbw_spmm_state;
 
 /* C may be NULL when beta == 0.  variant < 0 selects automatically. */
@@ -175,9 +176,15 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  *   reference's col2im, spconv/conv_format.h:77-81); Ho = (H + 2*(R/2) - R)/stride + 1.
  * Preconditions: filter synced, bcol == 1, C % 8 == 0, F % 8 == 0.
  * init allocates device scratch inside the filter object (freed with it; states made from one
- * filter with equal scratch size share it, so launch them on one stream); exec only launches:
- * im2col, the SpMM kernel, and the transpose to NHWC, in order on `stream`.
- * shflbw_spconv_init_variant: variant 0 = that pipeline, 1 = a single direct kernel.
+ * filter with equal scratch size share it, so launch them on one stream); exec only launches, in
+ * order on `stream`: a layout pass over the input, the SpMM kernel, and the transpose to NHWC.
+ * shflbw_spconv_init_variant:
+ *   variant 0 (default) = plane form: the input is rewritten once per call as channel-major padded
+ *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
+ *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,
+ *     its address generation is the per-id offset of the gather;
+ *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads);
+ *   variant 2 = explicit im2col matrix, SpMM, transpose.
  * ------------------------------------------------------------------------- */
 typedef struct shflbw_spconv_state {
     size_t shared_mem_size;
@@ -200,11 +207,17 @@ typedef struct shflbw_spconv_state {
     const int* packed_indices;
     const int* panel_ptr;
     int brow;
-    /* pipeline form (variant 0): im2col matrix [R*S*C][np] and filter-major result [F][np] in
-     * device scratch owned by the filter, np = B*Ho*Wo rounded up to 64; the SpMM launch state */
+    /* Device scratch owned by the filter and the state of the SpMM launch in the middle.
+     * Plane form (variant 0): `planes` holds the input as channel-major zero-padded planes
+     * [plane_copies][stride*stride][C][plane_pitch]; a "pixel" of the GEMM is a position
+     * b*plane_rows*plane_cols + i*plane_cols + j of that padded grid, np = B*plane_rows*plane_cols of
+     * them, and result_fm is [F][np].  im2col form (variant 2): im2col is the matrix [R*S*C][np],
+     * np = B*Ho*Wo rounded up to 64, result_fm [F][np]. */
     void* im2col;
     void* result_fm;
     int np;
+    void* planes;
+    int plane_rows, plane_cols, plane_pitch, plane_copies;
     shflbw_spmm_state spmm;
 } shflbw_spconv_state;
 

@@ -68,7 +68,8 @@ class SpconvState(C.Structure):
                 ("Ho", C.c_int), ("Wo", C.c_int),
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("panel_ptr", C.c_void_p),
                 ("brow", C.c_int), ("im2col", C.c_void_p), ("result_fm", C.c_void_p), ("np", C.c_int),
-                ("spmm", SpmmState)]
+                ("planes", C.c_void_p), ("plane_rows", C.c_int), ("plane_cols", C.c_int), ("plane_pitch", C.c_int),
+                ("plane_copies", C.c_int), ("spmm", SpmmState)]
 
 
 _lib = None

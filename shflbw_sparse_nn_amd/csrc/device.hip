@@ -6,6 +6,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "shflbw.h"
 #include "spconv_launch.h"
@@ -191,6 +192,7 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     state->packed_indices_pm = (const int*)w->d_packed_indices_pm;
     state->panel_ptr = (const int*)w->d_group_ptr;
     state->brow = w->brow;
+    state->ldb_bytes = N * 2;
     state->variant = variant;
     state->shared_mem_size = (size_t)v->lds_bytes;
     state->grid_dim[0] = (unsigned)(X * ((N + v->BN - 1) / v->BN));
@@ -227,6 +229,7 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
     a.panel_desc = state->panel_ptr;
     a.row_ids = state->args.A_row_indices;
     a.B = (const half_t*)state->args.B;
+    a.ldb_bytes = state->ldb_bytes;
     a.C = (const half_t*)state->args.C;
     a.D = (half_t*)state->args.D;
     a.alpha = state->args.alpha;
@@ -286,8 +289,8 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         set_error("spconv_init: empty output (%d x %d)", Ho, Wo);
         return SHFLBW_ERR_SHAPE;
     }
-    if (variant != 0 && variant != 1) {
-        set_error("spconv_init: variant %d does not exist (0 = pipeline, 1 = direct kernel)", variant);
+    if (variant < 0 || variant > 2) {
+        set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = im2col form)", variant);
         return SHFLBW_ERR_INVALID;
     }
     const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
@@ -324,23 +327,102 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     state->brow = f->brow;
     state->variant = variant;
     const long npix = (long)B * Ho * Wo;
+    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is not part of the weight's value
+    const int key[5] = {variant, B, H, W, stride};
+    auto cached_scratch = [&](size_t bytes, bool* fresh) -> void* {
+        for (auto& sc : fw->conv_scratch)
+            if (sc.bytes == bytes && memcmp(sc.key, key, sizeof(key)) == 0) {
+                *fresh = false;
+                return sc.ptr;
+            }
+        void* ptr = nullptr;
+        if (hipMalloc(&ptr, bytes) != hipSuccess) return nullptr;
+        shflbw_weight::Scratch sc{bytes, ptr, {key[0], key[1], key[2], key[3], key[4]}};
+        fw->conv_scratch.push_back(sc);
+        *fresh = true;
+        return ptr;
+    };
+    auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
     if (variant == 0) {
-        // pipeline form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
+        // plane form: geometry of the phase planes (see spconv_gfx950.hip)
+        const int s = stride, ph = f->R / 2, pw = f->S / 2;
+        const long PH = (H + 2 * ph + s - 1) / s;
+        const long PW = ((W + 2 * pw + s - 1) / s + 7) / 8 * 8;
+        const long np = (long)B * PH * PW;                                   // plane positions = GEMM columns
+        const long max_shift = (long)((f->R - 1) / s) * PW + (f->S - 1) / s; // largest tap offset
+        const long pitch = (np + max_shift + 8 + 63) / 64 * 64;
+        const int copies = (f->S - 1) / s >= 1 ? 2 : 1;
+        if (copies * s * s > 32) {
+            set_error("spconv_init: stride %d has too many phase planes for the plane form", s);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        const long rows = (long)copies * s * s * f->C; // channel rows of the plane tensor
+        if (np > 0x7fffffffL || (unsigned long long)rows * (unsigned long long)pitch * 2ull > 0xffffffffull) {
+            set_error("spconv_init: problem too large for the plane form (%ld rows of %ld positions)", rows, pitch);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        const size_t slots = f->packed_indices.size();
+        const size_t planes_bytes = up256((size_t)rows * pitch * 2), dm_bytes = up256((size_t)f->F * np * 2);
+        const size_t ids_bytes = up256(slots * sizeof(int) + 64);
+        bool fresh = false;
+        char* scratch = (char*)cached_scratch(planes_bytes + dm_bytes + 2 * ids_bytes, &fresh);
+        if (!scratch) {
+            set_error("spconv_init: cannot allocate %zu bytes of device scratch", planes_bytes + dm_bytes + 2 * ids_bytes);
+            return SHFLBW_ERR_HIP;
+        }
+        int* d_ids = (int*)(scratch + planes_bytes + dm_bytes);
+        int* d_ids_pm = (int*)(scratch + planes_bytes + dm_bytes + ids_bytes);
+        if (fresh) {
+            // the tail of every channel row and the positions no image covers are read (for results
+            // nobody uses) but never written
+            SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes));
+            // kept-column id k = (r*S + t)*C + c  ->  element offset of (copy, phase, channel) row + tap offset
+            std::vector<int> ids(slots), ids_pm(slots);
+            for (size_t q = 0; q < slots; q++) {
+                const int k = f->packed_indices[q];
+                const int c = k % f->C, tap = k / f->C, r = tap / f->S, t = tap % f->S;
+                const long shift = (long)(r / s) * PW + t / s;
+                const int copy = copies == 2 ? (int)(shift & 1) : 0;
+                const int phase = (r % s) * s + t % s;
+                ids[q] = (int)((((long)copy * s * s + phase) * f->C + c) * pitch + shift - copy);
+            }
+            for (size_t q = 0; q < slots; q++) { // producer-major order inside every 64-slot group
+                const size_t grp = q / 64;
+                const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
+                ids_pm[grp * 64 + 16 * p + 4 * j + r] = ids[q];
+            }
+            SHFLBW_HIP_TRY(hipMemcpy(d_ids, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+            SHFLBW_HIP_TRY(hipMemcpy(d_ids_pm, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+        }
+        state->planes = scratch;
+        state->result_fm = scratch + planes_bytes;
+        state->np = (int)np;
+        state->plane_rows = (int)PH;
+        state->plane_cols = (int)PW;
+        state->plane_pitch = (int)pitch;
+        state->plane_copies = copies;
+        int rc = shflbw_spmm_init(&state->spmm, f, (int)np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
+        if (rc != SHFLBW_OK) return rc;
+        // the gather walks the planes: ids are element offsets, one id apart is one value apart
+        state->spmm.packed_indices = d_ids;
+        state->spmm.packed_indices_pm = d_ids_pm;
+        state->spmm.ldb_bytes = 2;
+        state->spmm.args.K = (int)(rows * pitch); // extent of the id space
+    }
+    if (variant == 2) {
+        // im2col form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
         const long np = (npix + 63) / 64 * 64;
         const long K = (long)f->R * f->S * f->C;
         if (np > 0x7fffffffL || (unsigned long long)K * (unsigned long long)np * 2ull > 0xffffffffull) {
-            set_error("spconv_init: problem too large for the pipeline form (im2col matrix of %ld x %ld)", K, np);
+            set_error("spconv_init: problem too large for the im2col form (im2col matrix of %ld x %ld)", K, np);
             return SHFLBW_ERR_UNSUPPORTED;
         }
         const size_t bm_bytes = (size_t)K * np * 2, dm_bytes = (size_t)f->F * np * 2;
-        const size_t bytes = bm_bytes + dm_bytes;
-        shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is not part of the weight's value
-        void* scratch = nullptr;
-        for (auto& sc : fw->conv_scratch)
-            if (sc.bytes == bytes) scratch = sc.ptr;
+        bool fresh = false;
+        void* scratch = cached_scratch(bm_bytes + dm_bytes, &fresh);
         if (!scratch) {
-            SHFLBW_HIP_TRY(hipMalloc(&scratch, bytes));
-            fw->conv_scratch.push_back({bytes, scratch});
+            set_error("spconv_init: cannot allocate %zu bytes of device scratch", bm_bytes + dm_bytes);
+            return SHFLBW_ERR_HIP;
         }
         state->im2col = scratch;
         state->result_fm = (char*)scratch + bm_bytes;
@@ -393,6 +475,23 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
     if (state->variant == 0) {
+        hipError_t e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
+                                             state->plane_pitch, state->plane_copies, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: plane layout launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        int rc = shflbw_spmm_exec(&state->spmm, stream);
+        if (rc != SHFLBW_OK) return rc;
+        e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, state->np, a.B, state->plane_rows,
+                                  state->plane_cols, a.Ho, a.Wo, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: transpose launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        return SHFLBW_OK;
+    }
+    if (state->variant == 2) {
         hipError_t e = launch_im2col_nhwc(a, (half_t*)state->im2col, state->np, (hipStream_t)stream);
         if (e != hipSuccess) {
             set_error("spconv_exec: im2col launch failed: %s", hipGetErrorString(e));

@@ -158,7 +158,7 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
 
 
 // =======================================================================================
-// Pipeline form of the convolution (the default): three launches on the caller's stream
+// im2col form of the convolution: three launches on the caller's stream
 //   1. im2col_nhwc_kernel:   NHWC input -> im2col matrix Bm[k][p], k = (r,s,c), p = output pixel,
 //                            rows of NP fp16 (NP = pixel count rounded up to 64), zero outside the image
 //   2. the SpMM kernel:      Dm[f][p] = A_sparse * Bm (row permutation applied to f)
@@ -268,6 +268,109 @@ __global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __
             const int pix = p0 + o, f = f0 + q * 8;
             if (pix < npix && f < F) *(half8_t*)(out + (size_t)pix * F + f) = v;
         });
+}
+
+// =======================================================================================
+// Plane form of the convolution (the default): three launches on the caller's stream
+//   1. nhwc_to_planes_kernel: NHWC input -> channel-major, zero-padded planes.  With stride s the
+//      padded image is split into its s x s phases; phase (a, b) holds the padded positions
+//      (s i + a, s j + b) as a grid of PH x PW values (PW a multiple of 8), images back to back:
+//      position n' = img * PH * PW + i * PW + j.  One such row of `pitch` values per channel and
+//      phase.  A second copy of everything, moved by one value (copy[x] = base[x + 1]), serves the
+//      taps whose offset is odd, so that the gather below stays at least 4-byte aligned.
+//   2. the SpMM kernel over the positions n' as columns: the output pixel (ho, wo) of an image is
+//      the position (i, j) = (ho, wo), and tap (r, t) of channel c reads phase (r % s, t % s) of
+//      that channel at the constant offset (r / s) * PW + t / s.  The kept-column id of a vector is
+//      replaced by that element offset and the "row pitch" of B by one element: the im2col
+//      address generation is the offset of the gather, no im2col matrix exists.  Positions that
+//      are no output pixel (i >= Ho or j >= Wo) compute values nobody reads.
+//   3. planes_to_nhwc_kernel: Dm[f][n'] -> OFMap[pixel][f] for the positions that are pixels.
+// =======================================================================================
+struct PlaneGeom {
+    int B, H, W, C, stride, pad_h, pad_w;
+    int PH, PW;   // rows and (padded) columns of a phase plane
+    int pitch;    // values per channel row of the plane tensor
+    int copies;   // 1, or 2 with the copy moved by one value
+    int nwanted;  // (copy, phase) planes some tap reads; the others are never written
+    unsigned char wanted[32]; // copy * stride * stride + phase of each
+};
+
+// grid: (position tiles, channel tiles, wanted planes); block 256
+__global__ void __launch_bounds__(256) nhwc_to_planes_kernel(const half_t* __restrict__ in, half_t* __restrict__ planes,
+                                                             PlaneGeom g)
+{
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
+    const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT;
+    const int nphase = g.stride * g.stride;
+    const int copy = g.wanted[blockIdx.z] / nphase, phase = g.wanted[blockIdx.z] % nphase;
+    const int pa = phase / g.stride, pb = phase % g.stride;
+    const int PS = g.PH * g.PW;
+    half_t* dst = planes + ((size_t)(copy * nphase + phase) * g.C) * g.pitch;
+    transpose_tile_64(
+        tile,
+        [&](int i, int j) { // source row = position p0 + i (+ copy), piece = channels c0 + 8j ..
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            const int n = p0 + i + copy;
+            const int img = n / PS, rem = n % PS;
+            const int hi = (rem / g.PW) * g.stride + pa - g.pad_h, wi = (rem % g.PW) * g.stride + pb - g.pad_w;
+            const int c = c0 + j * 8;
+            if (img < g.B && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && c < g.C)
+                v = *(const half8_t*)(in + ((size_t)(img * g.H + hi) * g.W + wi) * g.C + c);
+            return v;
+        },
+        [&](int o, int q, half8_t v) { // destination row = channel c0 + o, positions p0 + 8q ..
+            if (c0 + o < g.C) *(half8_t*)(dst + (size_t)(c0 + o) * g.pitch + p0 + q * 8) = v;
+        });
+}
+
+// grid: (position tiles, filter tiles); block 256.  dm has rows of NP values.
+__global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __restrict__ dm, half_t* __restrict__ out, int F,
+                                                             int NP, int B, int PH, int PW, int Ho, int Wo)
+{
+    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
+    const int p0 = blockIdx.x * TT, f0 = blockIdx.y * TT;
+    const int PS = PH * PW;
+    transpose_tile_64(
+        tile,
+        [&](int i, int j) { // source row = filter f0 + i, piece = positions p0 + 8j ..
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (f0 + i < F && p0 + j * 8 < NP) v = *(const half8_t*)(dm + (size_t)(f0 + i) * NP + p0 + j * 8);
+            return v;
+        },
+        [&](int o, int q, half8_t v) { // destination row = the pixel at position p0 + o, filters f0 + 8q ..
+            const int n = p0 + o, f = f0 + q * 8;
+            const int img = n / PS, rem = n % PS, ho = rem / PW, wo = rem % PW;
+            if (img < B && ho < Ho && wo < Wo && f < F) *(half8_t*)(out + ((size_t)(img * Ho + ho) * Wo + wo) * F + f) = v;
+        });
+}
+
+hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int PH, int PW, int pitch, int copies,
+                                 hipStream_t stream)
+{
+    PlaneGeom g{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, PH, PW, pitch, copies, 0, {}};
+    // the planes the taps read: tap (r, t) -> phase (r % s, t % s), copy = parity of its offset when there are two
+    const int s = a.stride, nphase = s * s;
+    if (copies * nphase > (int)sizeof(g.wanted)) return hipErrorInvalidValue;
+    bool want[32] = {};
+    for (int r = 0; r < a.R; r++)
+        for (int t = 0; t < a.S; t++) {
+            const int shift = (r / s) * PW + t / s;
+            want[(copies == 2 ? (shift & 1) : 0) * nphase + (r % s) * s + t % s] = true;
+        }
+    for (int i = 0; i < copies * nphase; i++)
+        if (want[i]) g.wanted[g.nwanted++] = (unsigned char)i;
+    const int np = a.B * PH * PW;
+    const dim3 grid((np + TT - 1) / TT, (a.C + TT - 1) / TT, g.nwanted);
+    hipLaunchKernelGGL(nhwc_to_planes_kernel, grid, dim3(256), 0, stream, a.in, planes, g);
+    return hipGetLastError();
+}
+
+hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, int B, int PH, int PW, int Ho, int Wo,
+                                 hipStream_t stream)
+{
+    const dim3 grid((NP + TT - 1) / TT, (F + TT - 1) / TT);
+    hipLaunchKernelGGL(planes_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, NP, B, PH, PW, Ho, Wo);
+    return hipGetLastError();
 }
 
 hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream)

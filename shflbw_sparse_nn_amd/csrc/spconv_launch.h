@@ -29,7 +29,15 @@ struct SpconvVariant {
 
 const SpconvVariant* spconv_variants(int* count);
 
-// Stages 1 and 3 of the pipeline form of the convolution: NHWC input -> im2col matrix with rows of NP
+// Stages 1 and 3 of the plane form of the convolution: NHWC input -> channel-major padded planes (one per
+// stride phase, `copies` = 1 or 2 with a copy moved by one value, rows of `pitch` values), and the
+// filter-major result over plane positions (rows of NP values) -> NHWC output.
+hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int PH, int PW, int pitch, int copies,
+                                 hipStream_t stream);
+hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, int B, int PH, int PW, int Ho, int Wo,
+                                 hipStream_t stream);
+
+// Stages 1 and 3 of the im2col form of the convolution: NHWC input -> im2col matrix with rows of NP
 // halves (NP a multiple of 64), and filter-major result -> NHWC output.
 hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream);
 hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int npix, int NP, hipStream_t stream);

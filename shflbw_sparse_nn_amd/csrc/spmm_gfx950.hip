@@ -138,7 +138,8 @@ __global__ void __launch_bounds__(NWAVES * 64) spmm_shflbw_kernel(SpmmLaunchArgs
             int k = ks[j * RPI];
 #pragma unroll
             for (int q = 1; q < RPI; q++) k = (sub == q) ? ks[j * RPI + q] : k;
-            global_to_lds_16B(a.B + ((size_t)k * N + gcol[j]), sb + (wave * IPW + j) * 1024);
+            global_to_lds_16B((const half_t*)((const char*)a.B + (size_t)k * a.ldb_bytes) + gcol[j],
+                              sb + (wave * IPW + j) * 1024);
         }
     };
 
@@ -759,7 +760,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         //    start of the current group and first touched when that group is finished, several
         //    hundred cycles later, so the full wait a scalar load needs never stalls.
         const int pw = wave - NCONS;
-        const uint32_t rowbytes = (uint32_t)N * 2;
+        const uint32_t rowbytes = (uint32_t)a.ldb_bytes;
         const SHFLBW_CONST int2_t* desc = (const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc;
         constexpr int KSPS = Cfg::KSPS;
         constexpr int NSG = 64 / KT; // stages per group
@@ -919,7 +920,8 @@ static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
     b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
     const int T = a.X * b.n_tiles;
     // the gather addresses rows of B with 32-bit byte offsets
-    if ((unsigned long long)a.K * (unsigned long long)a.N * 2ull > 0xffffffffull) return hipErrorInvalidValue;
+    if ((unsigned long long)a.K * (unsigned long long)a.ldb_bytes + (unsigned long long)a.N * 2ull > 0xffffffffull)
+        return hipErrorInvalidValue;
     // one persistent workgroup per compute unit; fewer when there are fewer tiles (multiple of 8 XCDs)
     int grid = a.num_cus > 0 ? a.num_cus : 256;
     grid = (grid / 8) * 8;

@@ -15,6 +15,7 @@ struct SpmmLaunchArgs {
     const int* panel_desc;  // private image: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
     const int* row_ids;     // M, or null when rows are not permuted
     const half_t* B;
+    int ldb_bytes;          // bytes between rows of B one id apart (N * 2 for a dense row-major B)
     const half_t* C;
     half_t* D;
     float alpha, beta;

@@ -40,12 +40,14 @@ struct shflbw_weight {
     void* d_packed_indices_pm = nullptr;
     void* d_packed_values = nullptr;
 
-    // device scratch of the pipeline form of the convolution (im2col matrix followed by the
-    // filter-major result), one allocation per distinct size, handed out by shflbw_spconv_init
-    // and kept until the weight is re-initialised or destroyed
+    // device scratch of the multi-launch forms of the convolution (layout-transformed input, the
+    // filter-major result and, for the plane form, the kept-column ids rewritten as plane offsets),
+    // one allocation per distinct problem geometry, handed out by shflbw_spconv_init and kept until
+    // the weight is re-initialised or destroyed
     struct Scratch {
         size_t bytes;
         void* ptr;
+        int key[5]; // variant, B, H, W, stride
     };
     std::vector<Scratch> conv_scratch;
 };

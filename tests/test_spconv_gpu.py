@@ -19,7 +19,8 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    for variant in ((0, 1) if V != 16 else (0,)):  # 0: im2col + SpMM + transpose (default), 1: one direct kernel
+    # 0: plane layout + SpMM + transpose (default), 1: one direct kernel, 2: im2col matrix + SpMM + transpose
+    for variant in ((0, 1, 2) if V != 16 else (0, 2)):
         got = run_spconv(torch, w, R, S, C, x, stride, variant)
         assert got.shape == ref.shape
         assert not np.isnan(got.astype(np.float32)).any(), "variant %d left output elements unwritten" % variant
@@ -32,7 +33,10 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     (3, 9, 9, 8, 128, 1, 1, 1, 128, 0.6, False),  # 1x1 filter, no permutation
     (2, 8, 8, 24, 64, 5, 3, 1, 32, 0.2, True),    # rectangular filter
     (4, 14, 14, 64, 128, 3, 3, 2, 64, 0.05, True),
-    (2, 9, 7, 16, 48, 3, 3, 1, 16, 0.4, True),    # block height 16 (pipeline form only)
+    (2, 9, 7, 16, 48, 3, 3, 1, 16, 0.4, True),    # block height 16 (no direct kernel)
+    (2, 12, 10, 8, 64, 5, 5, 2, 32, 0.3, True),   # 5x5 stride 2: tap offsets 0..2 inside a phase plane
+    (1, 11, 9, 16, 64, 3, 3, 3, 64, 0.5, True),   # stride 3: nine phase planes, one tap each
+    (2, 6, 20, 8, 32, 1, 7, 1, 32, 0.4, True),    # 1x7 filter: seven tap offsets in one row
 ])
 def test_exact_shapes(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute):
     _exact(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute)
