@@ -46,6 +46,9 @@ def test_reference_case_all_variants(torch_gpu, V, permute):
     (1024, 1024, 1024, 64, 0.25),  # cfg0 shape
     (48, 72, 40, 16, 0.7),      # block height 16: three panels, ragged N and K
     (512, 1000, 513, 16, 0.15),
+    (33728, 1056, 128, 64, 0.05),  # tall weight of the reference's sweep list (527 panels, three column tiles)
+    (4096, 128, 512, 32, 0.1),     # N smaller than a column tile
+    (2048, 6400, 64, 64, 0.5),     # short panels (2 stages), many column tiles: tile switches dominate
 ])
 def test_exact_shapes(torch_gpu, M, N, K, V, d):
     _exact_case(torch_gpu, M, N, K, V, d, True)
