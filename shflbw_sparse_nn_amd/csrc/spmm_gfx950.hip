@@ -977,12 +977,12 @@ static hipError_t prepare_variant()
     }
 
 static const SpmmVariant g_variants[] = {
-    // block 64
-    SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
+    // block 64 (the first entry of a block size is the library's choice; measured order)
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 4),
+    SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
+    SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
     SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
-    SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 4),
     SHFLBW_VARIANT(64, 64, 4, 32, 3),
     SHFLBW_VARIANT(64, 64, 4, 32, 2),
@@ -993,6 +993,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(64, 32, 4, 32, 3),
     // block 32
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
+    SHFLBW_WS_VARIANT(32, 128, 4, 4, 32, 4),
     SHFLBW_VARIANT(32, 64, 4, 32, 3),
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
