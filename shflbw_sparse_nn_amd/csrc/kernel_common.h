@@ -84,6 +84,16 @@ __device__ __forceinline__ void wait_vmcnt_fence()
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
+// 16-byte store of result values with device scope: the line is written through to memory instead of
+// staying dirty in the XCD's L2, where its later eviction would fall into the gathers of the next tile.
+// The compiler has no form of this store, so it is inline assembly, and the compiler's hazard pass does
+// not look inside: a vector-ALU write to the data registers directly behind a store of more than 8 bytes
+// needs wait states, which the s_nop supplies (the registers are free for reuse after the statement).
+__device__ __forceinline__ void store_result_16B(half_t* p, half8_t v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+}
+
 // Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs; this makes consecutive *logical* ids share an XCD (and
 // therefore its L2), so tiles that gather the same activation slab run side by side.

@@ -546,7 +546,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
                                     v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
                         }
 #pragma unroll
-                        for (int it = 0; it < NIT; it++) *(half8_t*)(a.D + roff[it] + col) = v[it];
+                        for (int it = 0; it < NIT; it++) store_result_16B(a.D + roff[it] + col, v[it]);
                     }
                 }
             }
@@ -686,7 +686,7 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
                         for (int e = 0; e < 8; e++) v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
                 }
 #pragma unroll
-                for (int it = 0; it < 2; it++) *(half8_t*)(a.D + roff[it] + col) = v[it];
+                for (int it = 0; it < 2; it++) store_result_16B(a.D + roff[it] + col, v[it]);
             }
         }
     }
