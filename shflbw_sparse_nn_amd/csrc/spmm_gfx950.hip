@@ -1000,9 +1000,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(32, 64, 2, 32, 3),
     // block 16
     SHFLBW_WS_VARIANT(16, 128, 4, 4, 32, 4),
-    // block 128
-    SHFLBW_VARIANT(128, 64, 4, 32, 3),
-    SHFLBW_VARIANT(128, 32, 4, 32, 3),
+    // block 128 has no entries of its own: its panels are run as pairs of 64-row panels by the block-64 entries
 };
 
 const SpmmVariant* spmm_variants(int* count)

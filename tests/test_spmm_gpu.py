@@ -79,7 +79,7 @@ def test_empty_panels_write_zeros(torch_gpu):
     assert X == 4 and (got[np.sort(w["row_permute_ids"][:V])] == 0).all()
 
 
-@pytest.mark.parametrize("V", [16, 32])
+@pytest.mark.parametrize("V", [16, 32, 64, 128])
 @pytest.mark.parametrize("permute", [False, True])
 def test_beta_c_epilogue(torch_gpu, permute, V):
     # D = A*B + C, the overload the reference's example uses (example/spmm.blockwise.cu:50)
