@@ -177,7 +177,8 @@ def main():
     traffic = MEASURED_TRAFFIC.get((args.config, variant_name)) if args.traffic is None else float(args.traffic)
     traffic = None if traffic is None else round(traffic)
     out = {
-        "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64",
+        "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64" if args.config == "cfg1"
+                  else "effective sparse TFLOP/s + %% fp16 MFMA peak, SpMM %s" % args.config,
         "value": round(eff_tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -188,7 +189,8 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16 (fp32 accumulate)",
-        "data": "synthetic: seeded Shfl-BW mask + permutation (reference generators, seed 2021), values U[-1,1]",
+        "data": "synthetic: seeded Shfl-BW mask + permutation (reference generators, seed 2021), values A %s(%g), B %s(%g)"
+                % (c["a_dist"] + c["b_dist"]),
         "config": {"workload": "%s: Shfl-BW SpMM M=%d K=%d N=%d, block %d, density %g, row-permuted; nnzb=%d"
                                % (args.config, M, K, N, V, d, nnzb),
                    "kernel": variant_name, "timing": "events around %d back-to-back launches, operands resident"

@@ -992,8 +992,8 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(64, 64, 2, 32, 3),
     SHFLBW_VARIANT(64, 32, 4, 32, 3),
     // block 32
-    SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 32, 4),
+    SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
     SHFLBW_VARIANT(32, 64, 4, 32, 3),
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
