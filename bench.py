@@ -35,8 +35,9 @@ MEASURED_TRAFFIC = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=11)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500,
+                    help="untimed launches before the timed ones; the shader clock needs about 10 ms of load to settle")
     ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D)")
     ap.add_argument("--variant", type=int, default=-1, help="force a tile variant (default: library choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

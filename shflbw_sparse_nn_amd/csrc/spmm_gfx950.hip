@@ -794,13 +794,22 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
 
         // -- per-tile lane offsets: copy j of a stage fills row pw*RPW + j (swizzle key j % 4); the
         // lane's 16-byte piece lands at physical position `lane`, so it fetches logical piece lc
+        // -- direction: the workgroups of an XCD walk their tiles in step, all over the same columns of B.
+        // Every second tile of a workgroup is walked from its last stage to its first, so that a round of
+        // tiles starts on the rows of B the round before touched last (what is left of them in the
+        // XCD's L2) instead of on the ones it evicted first.  Only the order of the stages changes; inside
+        // a stage rows and A fragments stay as packed, and the consumers take the stages as they come.
+        bool rev = false;
         uint32_t voff[4];
         uint32_t va = 0;             // lane offset of this wave's A fragment of the next stage
+        uint32_t dva = 0;            // ... and its step from stage to stage
         const char* tileA = nullptr; // A fragments of the current tile
         auto open_tile = [&]() __attribute__((always_inline)) {
             const int n0 = (id / X) * BN;
             tileA = (const char*)a.packedA + (size_t)cur.y * (64 * V * 2);
-            va = pw * 1024 + lane * 16;
+            const int nst = (cur.x + KSPS - 1) / KSPS;
+            va = pw * 1024 + lane * 16 + (rev ? (uint32_t)(nst - 1) * (Cfg::A_FRAGS * 1024) : 0u);
+            dva = rev ? (uint32_t) - (Cfg::A_FRAGS * 1024) : (uint32_t)(Cfg::A_FRAGS * 1024);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
@@ -833,7 +842,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
                                  :
                                  : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
                                  : "m0", "scc");
-                va += Cfg::A_FRAGS * 1024;
+                va += dva;
                 sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
                                                                                        : sbp + STAGE_BYTES;
             };
@@ -847,6 +856,53 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             // load on them (it would otherwise wait, together with the loads of the following group,
             // at the top of every iteration)
             asm volatile("" : : "s"(gc0.x), "s"(gc1.x), "s"(gc2.x), "s"(gc3.x));
+            // stages of one group, first to last or last to first; a whole group is straight-line code
+            auto issue_group = [&](int n, bool back) __attribute__((always_inline)) {
+                if (KT == 16) { // four stages per group, stage j uses int4 j
+                    if (n == NSG && !back) {
+                        stage(gc0, gc0);
+                        stage(gc1, gc1);
+                        stage(gc2, gc2);
+                        stage(gc3, gc3);
+                    } else if (n == NSG) {
+                        stage(gc3, gc3);
+                        stage(gc2, gc2);
+                        stage(gc1, gc1);
+                        stage(gc0, gc0);
+                    } else if (!back) {
+                        stage(gc0, gc0);
+                        if (n > 1) stage(gc1, gc1);
+                        if (n > 2) stage(gc2, gc2);
+                    } else {
+                        if (n > 2) stage(gc2, gc2);
+                        if (n > 1) stage(gc1, gc1);
+                        stage(gc0, gc0);
+                    }
+                } else if (RPW == 8) { // two stages per group, stage j uses int4 2j and 2j + 1
+                    if (n == NSG && !back) {
+                        stage(gc0, gc1);
+                        stage(gc2, gc3);
+                    } else if (n == NSG) {
+                        stage(gc2, gc3);
+                        stage(gc0, gc1);
+                    } else {
+                        stage(gc0, gc1);
+                    }
+                } else { // two stages per group, stage j uses int4 j
+                    if (n == NSG && !back) {
+                        stage(gc0, gc0);
+                        stage(gc1, gc1);
+                    } else if (n == NSG) {
+                        stage(gc1, gc1);
+                        stage(gc0, gc0);
+                    } else {
+                        stage(gc0, gc0);
+                    }
+                }
+            };
+            auto groups_of = [&](int k16_steps) __attribute__((always_inline)) {
+                return ((k16_steps + KSPS - 1) / KSPS + NSG - 1) / NSG;
+            };
             while (true) {
                 const int nst = (cur.x + KSPS - 1) / KSPS; // stages of this tile
                 const int ngroups = (nst + NSG - 1) / NSG;
@@ -855,34 +911,16 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
                     have_next = true;
                 }
                 for (int q = 0; q < ngroups; q++) {
-                    const int n = min(NSG, nst - NSG * q);
-                    // the group that follows in the stream; at the very end simply this one again
-                    int gnext = cur.y + q + 1;
-                    if (q + 1 == ngroups) gnext = nxt.x > 0 ? nxt.y : cur.y + q;
+                    const int g = rev ? ngroups - 1 - q : q;                              // group of the tile
+                    const int n = g + 1 == ngroups ? nst - NSG * (ngroups - 1) : NSG;     // its stages
+                    // the group that follows in the stream (the next tile may be walked the other way round); at
+                    // the very end simply this one again
+                    int gnext = cur.y + (rev ? g - 1 : g + 1);
+                    if (q + 1 == ngroups)
+                        gnext = nxt.x > 0 ? nxt.y + ((rev != (a.alternate != 0)) ? groups_of(nxt.x) - 1 : 0) : cur.y + g;
                     const int4_t gn0 = *group_ptr(gnext, 0), gn1 = *group_ptr(gnext, 1), gn2 = *group_ptr(gnext, 2),
                                  gn3 = *group_ptr(gnext, 3);
-                    if (n == NSG) { // whole group: straight-line code
-                        if (KT == 16) {
-                            stage(gc0, gc0);
-                            stage(gc1, gc1);
-                            stage(gc2, gc2);
-                            stage(gc3, gc3);
-                        } else if (RPW == 8) {
-                            stage(gc0, gc1);
-                            stage(gc2, gc3);
-                        } else {
-                            stage(gc0, gc0);
-                            stage(gc1, gc1);
-                        }
-                    } else if (KT == 16) { // last, partial group of a tile
-                        stage(gc0, gc0);
-                        if (n > 1) stage(gc1, gc1);
-                        if (n > 2) stage(gc2, gc2);
-                    } else if (RPW == 8) {
-                        stage(gc0, gc1);
-                    } else {
-                        stage(gc0, gc0);
-                    }
+                    issue_group(n, rev);
                     if (!have_next) { // deferred from the start: not needed before the first copies are out
                         find_next();
                         have_next = true;
@@ -891,6 +929,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
                 }
                 if (nxt.x == 0) break;
                 id = idn, cur = nxt;
+                if (a.alternate) rev = !rev;
                 find_next();
                 open_tile();
             }

@@ -20,6 +20,8 @@ struct SpmmLaunchArgs {
     half_t* D;
     float alpha, beta;
     int num_cus; // compute units of the device (persistent kernels size their grid with it)
+    int alternate; // role-split kernels: walk every second tile of a workgroup from its last stage to its first
+                   // (pays when the rows of B under one column tile do not fit the XCD's L2)
 };
 
 struct SpmmVariant {

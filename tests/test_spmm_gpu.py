@@ -49,6 +49,12 @@ def test_reference_case_all_variants(torch_gpu, V, permute):
     (33728, 1056, 128, 64, 0.05),  # tall weight of the reference's sweep list (527 panels, three column tiles)
     (4096, 128, 512, 32, 0.1),     # N smaller than a column tile
     (2048, 6400, 64, 64, 0.5),     # short panels (2 stages), many column tiles: tile switches dominate
+    # more than 2.5 MB of B under a column tile and several tiles per workgroup: every second tile is
+    # walked from its last stage to its first (odd stage counts, partial last groups)
+    (8192, 1536, 4096, 32, 0.05),
+    (4096, 1024, 4096, 16, 0.03),
+    (8192, 2048, 3000, 64, 0.06),
+    (4096, 2048, 4096, 128, 0.07),
 ])
 def test_exact_shapes(torch_gpu, M, N, K, V, d):
     _exact_case(torch_gpu, M, N, K, V, d, True)
