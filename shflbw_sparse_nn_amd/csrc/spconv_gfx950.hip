@@ -417,7 +417,7 @@ static hipError_t prepare_conv()
 static const SpconvVariant g_conv_variants[] = {
     SHFLBW_CONV_VARIANT(64, 32, 4, 32),
     SHFLBW_CONV_VARIANT(32, 32, 4, 32),
-    // block 128: run as pairs of 64-row panels by the block-64 entry
+    SHFLBW_CONV_VARIANT(128, 32, 4, 32),
 };
 
 const SpconvVariant* spconv_variants(int* count)

@@ -286,10 +286,12 @@ struct SpmmWsCfg {
     // (32x32x16 tiles), V == 16 has one per 32-slot step (16x16x32 tiles)
     static constexpr int A_FRAGS = V == 16 ? KT / 32 : KSPS * MB;
     static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
-    static constexpr int RPW = KT / NPROD;                // gathered rows (= copies) per producer and stage
+    static constexpr int RPW = KT / NPROD;                // gathered rows per producer and stage
+    static constexpr int RPI = 1024 / ROWB;               // rows one 1 KiB copy instruction covers (BN = 256: two)
+    static constexpr int CPW = RPW / RPI;                 // copies of B rows per producer and stage
     static constexpr int A_HI = A_FRAGS % NPROD;          // producers [0, A_HI) copy one more A fragment
     static constexpr int A_LO = A_FRAGS / NPROD;
-    static constexpr int OPS = RPW + A_LO;                // copies per stage every producer issues at least
+    static constexpr int OPS = CPW + A_LO;                // copies per stage every producer issues at least
     static constexpr int EPI_ROWB = 32 * 2 + 16;
     static constexpr int EPI_ROWS = NCONS > 4 ? 16 : 32;  // rows of a 32 x 32 accumulator block staged at a time
     static constexpr int EPI_WAVE_BYTES = EPI_ROWS * EPI_ROWB;
@@ -297,16 +299,16 @@ struct SpmmWsCfg {
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
     static_assert((V % 32 == 0 || (V == 16 && KT == 32)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
-    static_assert(BN == 512, "one gathered row is exactly one 1 KiB copy instruction");
+    static_assert(BN == 512 || (BN == 256 && RPW == 8), "a 1 KiB copy instruction covers one gathered row, or two");
     static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
-    static_assert(A_LO <= 1 && (A_LO == 0 || A_HI == 0), "at most one A fragment per producer and stage");
+    static_assert(A_LO <= 2 && (A_LO == 0 || A_HI == 0), "the same number of A fragments for all producers that copy any");
     // A producer passes one barrier before every stage it issues.  The barrier in front of stage j is the
     // one after which the consumers no longer read stage j - NSTAGE, i.e. their barrier number j - (NSTAGE-2):
     // the consumers therefore pass NSTAGE - 2 extra barriers before their first one.
     static constexpr int START_BARRIERS = NSTAGE - 2;
     static_assert(THREADS <= 1024, "workgroup size limit");
     static_assert(NSTAGE >= 3, "one stage computed, one landed, one in flight");
-    static_assert((NSTAGE - 3) * (RPW + 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert((NSTAGE - 3) * (CPW + (A_LO > 0 ? A_LO : 1)) < 64, "vmcnt is a 6-bit counter");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 };
 
@@ -812,7 +814,11 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             dva = rev ? (uint32_t) - (Cfg::A_FRAGS * 1024) : (uint32_t)(Cfg::A_FRAGS * 1024);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int lc = ((((lane >> 1) ^ row_xor32(j))) << 1) | (lane & 1);
+                // one copy = one row of 64 pieces (swizzle key j % 4), or the rows 2j and 2j + 1 of this
+                // producer, 32 pieces each, in the lower and the upper half of the wave
+                const int key = Cfg::RPI == 1 ? j : (2 * j + (lane >> 5)) & 3;
+                const int pc = Cfg::RPI == 1 ? lane : lane & 31;
+                const int lc = ((((pc >> 1) ^ row_xor32(key))) << 1) | (pc & 1);
                 const int col = n0 + lc * 8;
                 voff[j] = (uint32_t)(col < N ? col : 0) * 2; // columns past N are never stored
             }
@@ -822,10 +828,12 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
         // fragment per stage: its copies per stage are then a compile-time number and the waits exact
         auto run = [&](auto has_a_tag) __attribute__((always_inline)) {
             constexpr bool HAS_A = decltype(has_a_tag)::value;
-            constexpr int MYOPS = RPW + (HAS_A ? 1 : 0); // copies per stage of this producer
+            constexpr int NA = HAS_A ? (Cfg::A_LO > 0 ? Cfg::A_LO : 1) : 0; // A fragments per stage of this producer
+            constexpr int MYOPS = Cfg::CPW + NA;                            // its copies per stage
             // ring position of the next stage: LDS address of this wave's rows
-            uint32_t sbp = lds0 + pw * RPW * 1024;
-            const int a_rel = B_BYTES + pw * 1024 - pw * RPW * 1024; // this wave's A fragment slot relative to sbp
+            uint32_t sbp = lds0 + pw * RPW * Cfg::ROWB;
+            // this wave's first A fragment slot relative to sbp (a second one lies NPROD fragments further)
+            const int a_rel = B_BYTES + pw * 1024 - pw * RPW * Cfg::ROWB;
             // One stage, branch-free: the barrier in front of stage j tells that the consumers are done with
             // the ring slot it overwrites; before arriving there the stage the consumers read next (issued
             // NSTAGE - 2 stages ago) must have landed, NSTAGE - 3 younger stages stay in flight.  In front
@@ -833,8 +841,17 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
             auto stage = [&](int4_t ka, int4_t kb) __attribute__((always_inline)) {
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * MYOPS));
                 wg_barrier();
-                gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
-                if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
+                if (Cfg::RPI == 1) {
+                    gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
+                    if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
+                } else {
+                    // 512-byte rows: the lower half of the wave fetches row 2j, the upper half row 2j + 1
+                    const bool hi = lane >= 32;
+                    global_to_lds_16B_sbase<0x000>(a.B, (uint32_t)(hi ? ka.y : ka.x) * rowbytes + voff[0], sbp);
+                    global_to_lds_16B_sbase<0x400>(a.B, (uint32_t)(hi ? ka.w : ka.z) * rowbytes + voff[1], sbp);
+                    global_to_lds_16B_sbase<0x800>(a.B, (uint32_t)(hi ? kb.y : kb.x) * rowbytes + voff[2], sbp);
+                    global_to_lds_16B_sbase<0xc00>(a.B, (uint32_t)(hi ? kb.w : kb.z) * rowbytes + voff[3], sbp);
+                }
                 if (HAS_A)
                     asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
                                  "s_nop 0\n\t"
@@ -842,9 +859,16 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(Sp
                                  :
                                  : [sbp] "s"(sbp), [arel] "s"(a_rel), [va] "v"(va), [A] "s"(tileA)
                                  : "m0", "scc");
+                if (NA == 2) // its second fragment, NPROD fragments further in memory and in the stage
+                    asm volatile("s_add_i32 m0, %[sbp], %[arel]\n\t"
+                                 "s_nop 0\n\t"
+                                 "global_load_lds_dwordx4 %[va], %[A]"
+                                 :
+                                 : [sbp] "s"(sbp), [arel] "s"(a_rel + NPROD * 1024), [va] "v"(va), [A] "s"(tileA + NPROD * 1024)
+                                 : "m0", "scc");
                 va += dva;
-                sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * 1024 + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
-                                                                                       : sbp + STAGE_BYTES;
+                sbp = (sbp + STAGE_BYTES == lds0 + pw * RPW * Cfg::ROWB + Cfg::RING_BYTES) ? sbp - (NSTAGE - 1) * STAGE_BYTES
+                                                                                            : sbp + STAGE_BYTES;
             };
 
             // -- groups: gc* = ids of the group being issued, gn* = ids of the group after it in the
@@ -1019,6 +1043,7 @@ static const SpmmVariant g_variants[] = {
     // block 64 (the first entry of a block size is the library's choice; measured order)
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 5),
+    SHFLBW_WS_VARIANT(64, 64, 4, 4, 32, 6),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 6),
     SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
@@ -1033,13 +1058,18 @@ static const SpmmVariant g_variants[] = {
     // block 32
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
+    SHFLBW_WS_VARIANT(32, 64, 4, 4, 32, 6),
     SHFLBW_VARIANT(32, 64, 4, 32, 3),
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
     SHFLBW_VARIANT(32, 64, 2, 32, 3),
     // block 16
     SHFLBW_WS_VARIANT(16, 128, 4, 4, 32, 4),
-    // block 128 has no entries of its own: its panels are run as pairs of 64-row panels by the block-64 entries
+    // block 128
+    SHFLBW_WS_VARIANT(128, 64, 4, 4, 32, 6),
+    SHFLBW_WS_VARIANT(128, 64, 4, 4, 32, 5),
+    SHFLBW_VARIANT(128, 64, 4, 32, 3),
+    SHFLBW_VARIANT(128, 32, 4, 32, 3),
 };
 
 const SpmmVariant* spmm_variants(int* count)

@@ -199,8 +199,7 @@ static int check_pattern(int nrow, int ncol, int brow, int bcol, int nnzb, const
 // values are zero).  packed_values: per MFMA k-step, the A operand in register
 // order, so one wave reads a fragment as 64 consecutive 16-byte pieces:
 //   V >= 32 (32x32x16 tiles): step s covers slots 16s..16s+15; block mb covers rows
-//     32mb..32mb+31; lane l holds row 32mb + l%32, slots 16s + 8*(l/32) + 0..7.  V == 128 is
-//     laid out as two 64-row panels with the same ids (kernel_block_rows).
+//     32mb..32mb+31; lane l holds row 32mb + l%32, slots 16s + 8*(l/32) + 0..7.
 //   V == 16 (16x16x32 tiles): step s covers slots 32s..32s+31; lane l holds row l%16,
 //     slots 32s + 8*(l/16) + 0..7.
 // ---------------------------------------------------------------------------------
@@ -215,26 +214,23 @@ int build_packed_image(shflbw_weight* w)
         set_error("no gfx950 kernel for block size %d (16, 32, 64, 128 are built)", V);
         return SHFLBW_ERR_UNSUPPORTED;
     }
-    // kernel panels: KV rows each, H of them per panel of the format (H = 2 for V = 128, else 1)
-    const int KV = kernel_block_rows(V), H = V / KV;
-    const int X = w->nrow / KV;
+    const int X = w->nrow / V;
     w->group_ptr.assign(X + 1, 0);
     for (int i = 0; i < X; i++) {
-        int nnz = w->indptr[i / H + 1] - w->indptr[i / H];
+        int nnz = w->indptr[i + 1] - w->indptr[i];
         w->group_ptr[i + 1] = w->group_ptr[i] + (nnz + 63) / 64;
     }
     w->panel_desc.assign(2 * (size_t)X, 0);
     for (int i = 0; i < X; i++) {
-        w->panel_desc[2 * i] = (w->indptr[i / H + 1] - w->indptr[i / H] + 15) / 16;
+        w->panel_desc[2 * i] = (w->indptr[i + 1] - w->indptr[i] + 15) / 16;
         w->panel_desc[2 * i + 1] = w->group_ptr[i];
     }
     const size_t slots = (size_t)w->group_ptr[X] * 64;
     w->packed_indices.assign(slots, 0);
     w->packed_indices_pm.assign(slots, 0);
-    w->packed_values.assign(slots * KV, 0);
+    w->packed_values.assign(slots * V, 0);
     for (int i = 0; i < X; i++) {
-        const int begin = w->indptr[i / H], nnz = w->indptr[i / H + 1] - begin;
-        const int row0 = (i % H) * KV; // first row, inside the format's panel, of this kernel panel
+        const int begin = w->indptr[i], nnz = w->indptr[i + 1] - begin;
         const size_t slot0 = (size_t)w->group_ptr[i] * 64;
         const int padded = (w->group_ptr[i + 1] - w->group_ptr[i]) * 64;
         for (int q = 0; q < padded; q++)
@@ -243,13 +239,13 @@ int build_packed_image(shflbw_weight* w)
             const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, r = q % 4;
             w->packed_indices_pm[slot0 + grp * 64 + 16 * p + 4 * j + r] = w->packed_indices[slot0 + q];
         }
-        uint16_t* dst = w->packed_values.data() + slot0 * KV;
-        const uint16_t* src = w->values.data() + (size_t)begin * V + row0;
-        if (KV >= 32) {
-            const int MB = KV / 32;
+        uint16_t* dst = w->packed_values.data() + slot0 * V;
+        const uint16_t* src = w->values.data() + (size_t)begin * V;
+        if (V >= 32) {
+            const int MB = V / 32;
             for (int q = 0; q < nnz; q++) {
                 const int s = q / 16, half_k = (q % 16) / 8, j = q % 8;
-                for (int r = 0; r < KV; r++) {
+                for (int r = 0; r < V; r++) {
                     const int mb = r / 32, lane = half_k * 32 + r % 32;
                     dst[(((size_t)s * MB + mb) * 64 + lane) * 8 + j] = src[(size_t)q * V + r];
                 }

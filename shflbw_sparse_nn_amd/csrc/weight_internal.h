@@ -23,7 +23,7 @@ struct shflbw_weight {
     std::vector<int> meta_h;
 
     // private image for the gfx950 kernels, built by sync_device
-    std::vector<int> group_ptr;      // X+1: cumulative count of 64-slot groups per kernel panel (X = nrow / kernel_block_rows)
+    std::vector<int> group_ptr;      // X+1: cumulative count of 64-slot groups per panel
     std::vector<int> panel_desc;     // 2X: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
     std::vector<int> packed_indices; // 64 * group_ptr[X]; tail slots repeat the panel's last id
     std::vector<int> packed_indices_pm; // each 64-slot group reordered: [16p + 4j + r] = packed_indices[16j + 4p + r]
@@ -59,11 +59,6 @@ void set_error(const char* fmt, ...);
 // fp16 bit helpers (IEEE binary16, round to nearest even)
 float half_to_float(uint16_t h);
 uint16_t float_to_half(float f);
-
-// Rows per panel as the kernels see them.  A panel of 128 rows is run as two panels of 64 rows that
-// keep the same columns (the private image repeats the ids and splits the values): stored row
-// 128 p + 64 h + r is row r of kernel panel 2 p + h, so the permutation array is indexed the same way.
-inline int kernel_block_rows(int brow) { return brow == 128 ? 64 : brow; }
 
 // k-extent of one MFMA step for a block size: 32x32x16 tiles for V >= 32, 16x16x32 for V == 16
 inline int mfma_kstep(int brow) { return brow >= 32 ? 16 : 32; }
