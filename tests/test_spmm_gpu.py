@@ -55,9 +55,22 @@ def test_reference_case_all_variants(torch_gpu, V, permute):
     (4096, 1024, 4096, 16, 0.03),
     (8192, 2048, 3000, 64, 0.06),
     (4096, 2048, 4096, 128, 0.07),
+    (4096, 4096, 8192, 128, 0.05),  # 128 x 256 tiles, two per workgroup, the second walked backwards
 ])
 def test_exact_shapes(torch_gpu, M, N, K, V, d):
     _exact_case(torch_gpu, M, N, K, V, d, True)
+
+
+@pytest.mark.parametrize("V", [32, 64])
+def test_narrow_tiles_on_a_large_problem(torch_gpu, V):
+    # the 256-column role-split variant is the library's choice for small problems only; forced here on a
+    # problem with two to four tiles per workgroup and 3 MB of B under a column tile (backwards walk on)
+    names = S.spmm_variants(V)
+    narrow = [i for i, n in enumerate(names) if n.startswith("ws%dx64x4c4p" % V)]
+    assert narrow, names
+    for variant in narrow:
+        print("variant", variant, names[variant], flush=True)
+        _exact_case(torch_gpu, 4096, 2048, 6144, V, 0.06, True, variant)
 
 
 def test_dense_density_is_permuted_gemm(torch_gpu):
