@@ -112,14 +112,16 @@ static const SpconvVariant* find_spconv_variant(int brow, int variant, int* n_fo
 // there, 5-20 % slower once the wide tiles fill the chip).
 static int auto_spmm_variant(int brow, int X, int N)
 {
+    const SpmmVariant* first = find_spmm_variant(brow, 0, nullptr);
+    if (!first || first->BN != 512) return 0;
     const long wide_tiles = (long)X * ((N + 511) / 512);
     if (wide_tiles > device_compute_units() / 2) return 0;
     int count = 0, seen = 0;
     const SpmmVariant* all = spmm_variants(&count);
-    if (!(find_spmm_variant(brow, 0, nullptr) && find_spmm_variant(brow, 0, nullptr)->BN == 512)) return 0;
     for (int i = 0; i < count; i++) {
         if (all[i].V != brow) continue;
-        if (all[i].BN == 256 && all[i].threads == 512 && all[i].name[0] == 'w') return seen;
+        const bool role_split = all[i].name[0] == 'w'; // "ws..." names
+        if (role_split && all[i].BN == 256) return seen;
         seen++;
     }
     return 0;
