@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
-"""Headline benchmark: Shfl-BW SpMM, M = K = N = 4096, block size 64, density 0.1, row-permuted
-(BASELINE.json configs[1]) on one MI355X.
+"""Benchmark of the Shfl-BW hot path on one MI355X.  Default workload: the headline SpMM, M = K = N = 4096,
+block size 64, density 0.1, row-permuted (BASELINE.json configs[1]).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg0|cfg1|cfg2|cfg3|cfg4]
 
-A step is one launch of the SpMM on device-resident operands (fp16 in, fp32 accumulate, fp16 out).
-Timing follows the reference's benchmark (benchmark/benchmark.spmm.cu:29-50): warm-up launches, then K
-back-to-back launches between two events on the launch stream; mean per launch.  Prints one JSON line:
-effective sparse TFLOP/s (2 * nnzb * V * N / t), the HBM roofline of the kernel, the dense fp16 GEMM of
-the same shape as a reference point, and the CPU oracle timed on the host cores as a baseline.
+A step is one `exec` of the operator on device-resident operands (fp16 in, fp32 accumulate, fp16 out):
+one launch for the SpMM configs (cfg0-cfg2), the whole convolution for cfg3/cfg4.  Timing follows the
+reference's benchmark (benchmark/benchmark.spmm.cu:29-50, benchmark.spconv.cu:29-50): warm-up launches,
+then K back-to-back launches between two events on the launch stream; mean per launch.  Prints one JSON
+line: effective sparse TFLOP/s (2 * nnzb * V * N / t), the roofline of the kernel, and the CPU oracle timed
+on the host cores as a baseline; the SpMM line also carries a dense fp16 GEMM of the same shape.
 """
 import argparse
 import json
@@ -23,13 +24,89 @@ if ROOT not in sys.path:
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix-core peak
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 
-# HBM-side bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs of this
-# script, each scaled by what the same counter reads for a 32 MiB device copy); keyed by
-# (config, kernel variant).  The summaries are kept under profiles/.
-MEASURED_TRAFFIC = {
-    ("cfg1", "ws64x128x4c4p_k32_s4"): 38094.4 * 1024 * 2.0 + 32768.0 * 1024 * 1.0,
-    ("cfg1", "ws64x128x4c4p_k16_s6"): 45972.9 * 1024 * 2.0 + 32772.9 * 1024 * 1.0,
-}
+
+def measured_traffic(config, kernel):
+    """HBM-side bytes per step from the tracked counter summary (profiles/traffic.json: FETCH_SIZE and
+    WRITE_SIZE runs of this script under rocprofv3 --pmc, each scaled by what the same counter reads for a
+    device copy of known size).  An entry only applies to the kernel it names; None when there is none."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        table = json.load(f)
+    for e in table.get("entries", []):
+        if e["config"] == config and e["kernel"] == kernel:
+            return round(e["fetch_kib"] * 1024 * e["fetch_scale"] + e["write_kib"] * 1024 * e["write_scale"])
+    return None
+
+
+def time_launches(torch, stream, op, n):
+    """Mean milliseconds of n back-to-back launches of `op` between two events on `stream`."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(n):
+        op(stream.cuda_stream)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n
+
+
+def reference_loop(torch, stream, op):
+    """The reference's own loop (1 + 10 warm-ups, 100 launches) from an idle GPU: the clock is still ramping."""
+    torch.cuda.synchronize()
+    time.sleep(0.05)
+    for _ in range(11):
+        op(stream.cuda_stream)
+    return time_launches(torch, stream, op, 100)
+
+
+def timed_region(torch, stream, op, steps, warmup):
+    for _ in range(warmup):
+        op(stream.cuda_stream)
+    torch.cuda.synchronize()
+    wall0 = time.time()
+    ms = time_launches(torch, stream, op, steps)
+    return ms, time.time() - wall0
+
+
+def roofline(eff_flops, alg_bytes, t, traffic):
+    """The bound of the workload (MFMA when its arithmetic intensity is above the ridge, else HBM) and the
+    fraction of it reached in t seconds."""
+    ai = eff_flops / alg_bytes
+    if ai * HBM_PEAK_GBS * 1e9 > MFMA_F16_PEAK_TFLOPS * 1e12:
+        a = eff_flops / t / 1e12
+        r = {"bound": "mfma", "achieved": round(a, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": round(a / MFMA_F16_PEAK_TFLOPS, 4)}
+    else:
+        a = alg_bytes / t / 1e9
+        r = {"bound": "hbm", "achieved": round(a, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(a / HBM_PEAK_GBS, 4)}
+    r.update({"traffic": traffic, "algorithmic_bytes": alg_bytes, "effective_flops": eff_flops})
+    return r
+
+
+def cpu_baseline(run_all, run_one, eff_flops, sub_flops, what_all, what_one, threads):
+    """The oracle (a port of the reference's get_host_reference) on the host cores: about 10 s with every
+    core on the whole workload, about 5 s with a single thread on a sample of it."""
+    run_all()  # page in
+    reps, t_sum = 0, 0.0
+    while t_sum < 10.0 and reps < 400:
+        t0 = time.time()
+        run_all()
+        t_sum += time.time() - t0
+        reps += 1
+    t_all = t_sum / reps
+    reps1, t1_sum = 0, 0.0
+    while t1_sum < 5.0 and reps1 < 200:
+        t0 = time.time()
+        run_one()
+        t1_sum += time.time() - t0
+        reps1 += 1
+    t_one = t1_sum / reps1
+    return {"value": round(eff_flops / t_all / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%s on %d threads, mean of %d runs (%.1f s of CPU work): %.4f s per pass; one thread on %s, "
+                      "mean of %d runs: %.4f s = %.4f TFLOP/s"
+                      % (what_all, threads, reps, t_sum, t_all, what_one, reps1, t_one, sub_flops / t_one / 1e12)}
 
 
 def main():
@@ -39,11 +116,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=500,
                     help="untimed launches before the timed ones; the shader clock needs about 10 ms of load to settle")
     ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D)")
-    ap.add_argument("--variant", type=int, default=-1, help="force a tile variant (default: library choice)")
+    ap.add_argument("--variant", type=int, default=-1, help="force a kernel variant (default: library choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--traffic", default=None,
-                    help="HBM bytes per launch from a newer rocprofv3 --pmc measurement; default: the committed "
-                         "figure for this config and kernel variant, null if there is none")
+                    help="HBM bytes per step from a newer rocprofv3 --pmc measurement; default: the tracked "
+                         "figure for this config and kernel, null if there is none")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -53,13 +130,17 @@ def main():
     import torch
 
     import shflbw_sparse_nn_amd as S  # raises if the HIP library is missing: there is no fallback
-    from tests import problems as P
-    from tests.gpu_util import to_dev, upload_weight
+    import workloads as P
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     if args.config in P.CONV_CONFIGS:
         return bench_conv(args, np, torch, S, P)
+    return bench_spmm(args, np, torch, S, P)
+
+
+def bench_spmm(args, np, torch, S, P):
+    from oracle import oracle as O  # correctness gate and CPU baseline only
     c = P.SPMM_CONFIGS[args.config]
     M, K, N, V, d = c["M"], c["K"], c["N"], c["V"], c["d"]
     w = P.make_weight(M, K, V, d, True, 2021, dist=c["a_dist"])
@@ -69,8 +150,8 @@ def main():
     # algorithmic bytes of one launch: A values + (indices, indptr, perm) + B once + D once
     alg_bytes = nnzb * V * 2 + (nnzb + M // V + 1 + M) * 4 + K * N * 2 + M * N * 2
 
-    mat = upload_weight(w)
-    dB = to_dev(torch, B)
+    mat = P.upload_weight(w)
+    dB = P.to_dev(torch, B)
     dD = torch.zeros((M, N), dtype=torch.float16, device="cuda")
     op = S.SpmmBlockwiseOp(args.variant)
     st = op.initialize(mat, N, dB.data_ptr(), dD.data_ptr())
@@ -78,67 +159,31 @@ def main():
     stream = torch.cuda.current_stream()
 
     # correctness gate before any timing: bit-exact against the oracle on the integer twin of the workload
-    from oracle import oracle as O
     wi = P.make_weight(M, K, V, d, True, 2021, integer=True)
     Bi = P.make_dense(K, N, 2021, integer=True)
-    mi = upload_weight(wi)
-    dBi = to_dev(torch, Bi)
+    mi = P.upload_weight(wi)
+    dBi = P.to_dev(torch, Bi)
     dDi = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     opi = S.SpmmBlockwiseOp(args.variant)
     opi.initialize(mi, N, dBi.data_ptr(), dDi.data_ptr())
     opi(stream.cuda_stream)
     torch.cuda.synchronize()
-    t0 = time.time()
     ref_i = O.float_to_half(P.spmm_oracle(wi, Bi))
-    t_oracle_all = time.time() - t0
     if not np.array_equal(dDi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
         print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
         sys.exit(1)
 
-    # ---- the reference's own loop first (benchmark/benchmark.spmm.cu:29-50: 1 + 10 warm-ups, 100 launches),
-    # from an idle GPU as its program sees it: the shader clock is still ramping up in these 2 ms
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(11):
-        op(stream.cuda_stream)
-    e0.record(stream)
-    for _ in range(100):
-        op(stream.cuda_stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ref_loop_ms = e0.elapsed_time(e1) / 100
-
-    # ---- timed region (events on the stream the kernel is launched on)
-    for _ in range(args.warmup):
-        op(stream.cuda_stream)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    wall0 = time.time()
-    e0.record(stream)
-    for _ in range(args.steps):
-        op(stream.cuda_stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall = time.time() - wall0
-    ms_per_step = e0.elapsed_time(e1) / args.steps
+    ref_loop_ms = reference_loop(torch, stream, op)
+    ms_per_step, wall = timed_region(torch, stream, op, args.steps, args.warmup)
     t = ms_per_step * 1e-3
     eff_tflops = eff_flops / t / 1e12
-    achieved_gbs = alg_bytes / t / 1e9
-
-    # ---- the same launch on the integer twin (values of the reference's generator, rand() % 9 - 4): the
-    # shader clock under MFMA load depends on the operand values, so this is reported beside the graded figure
-    for _ in range(args.warmup):
-        opi(stream.cuda_stream)
-    torch.cuda.synchronize()
-    e0.record(stream)
-    for _ in range(args.steps):
-        opi(stream.cuda_stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    int_ms = e0.elapsed_time(e1) / args.steps
+    # the same launch on the integer twin (values of the reference's generator, rand() % 9 - 4): the shader clock
+    # under MFMA load depends on the operand values, so this is reported beside the graded figure
+    int_ms, _ = timed_region(torch, stream, opi, args.steps, args.warmup)
     del mi, dBi, dDi, opi
 
     # ---- cold-cache variant: rotate operand sets larger than the 256 MB last-level cache
-    nsets = 5
+    nsets = max(2, min(8, int(320e6 // (2 * (K * N + M * N))) + 1))
     Bs = [dB] + [dB.clone() for _ in range(nsets - 1)]
     Ds = [dD] + [torch.zeros_like(dD) for _ in range(nsets - 1)]
     ops = []
@@ -149,6 +194,7 @@ def main():
     for i in range(nsets):
         ops[i](stream.cuda_stream)
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for i in range(args.steps):
         ops[i % nsets](stream.cuda_stream)
@@ -169,38 +215,17 @@ def main():
     torch.cuda.synchronize()
     dense_ms = e0.elapsed_time(e1) / 20
 
-    # ---- CPU baseline: the oracle (a port of the reference's get_host_reference) on the host cores, on the
-    # same workload; one run with every core, one with a single thread on a 1/8 sample of the row panels
     cpu = None
     if not args.no_cpu:
-        threads = O.max_threads()
-        P.spmm_oracle(w, B)  # page in
-        reps, t_sum = 0, 0.0
-        while t_sum < 10.0 and reps < 400:
-            t0 = time.time()
-            P.spmm_oracle(w, B)
-            t_sum += time.time() - t0
-            reps += 1
-        t_all = t_sum / reps
         X = M // V
-        sub = dict(w, nrow=(X // 8) * V, indptr=w["indptr"][:X // 8 + 1],
-                   indices=w["indices"][:w["indptr"][X // 8]], values=w["values"][:w["indptr"][X // 8] * V],
-                   row_permute_ids=None)
-        reps1, t1_sum = 0, 0.0
-        while t1_sum < 5.0 and reps1 < 200:
-            t0 = time.time()
-            P.spmm_oracle(sub, B, nthreads=1)
-            t1_sum += time.time() - t0
-            reps1 += 1
-        t_one = t1_sum / reps1
-        sub_flops = 2.0 * int(w["indptr"][X // 8]) * V * N
-        cpu = {"value": round(eff_flops / t_all / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-               "sample": "whole workload (%d panels) on %d threads, mean of %d runs (%.1f s of CPU work): %.4f s per "
-                         "pass; one thread on the first %d panels, mean of %d runs: %.4f s = %.4f TFLOP/s"
-                         % (X, threads, reps, t_sum, t_all, X // 8, reps1, t_one, sub_flops / t_one / 1e12)}
+        XS = max(1, X // 8)
+        sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
+                   values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
+        cpu = cpu_baseline(lambda: P.spmm_oracle(w, B), lambda: P.spmm_oracle(sub, B, nthreads=1), eff_flops,
+                           2.0 * int(w["indptr"][XS]) * V * N, "whole workload (%d panels)" % X,
+                           "the first %d panels" % XS, O.max_threads())
 
-    traffic = MEASURED_TRAFFIC.get((args.config, variant_name)) if args.traffic is None else float(args.traffic)
-    traffic = None if traffic is None else round(traffic)
+    traffic = measured_traffic(args.config, variant_name) if args.traffic is None else round(float(args.traffic))
     out = {
         "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64" if args.config == "cfg1"
                   else "effective sparse TFLOP/s + %% fp16 MFMA peak, SpMM %s" % args.config,
@@ -228,9 +253,7 @@ def main():
                                     "ms_per_step": round(int_ms, 6),
                                     "tflops": round(eff_flops / (int_ms * 1e-3) / 1e12, 1)},
         "dense_equivalent_tflops": round(2.0 * M * N * K / t / 1e12, 1),
-        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "algorithmic_bytes": alg_bytes, "effective_flops": eff_flops},
+        "roofline": roofline(eff_flops, alg_bytes, t, traffic),
         "cold_cache_ms_per_step": round(cold_ms, 6),
         "dense_gemm": {"what": "torch.matmul fp16 %dx%dx%d (hipBLASLt/rocBLAS)" % (M, N, K),
                        "ms": round(dense_ms, 6), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 1)},
@@ -242,21 +265,21 @@ def main():
 
 
 def bench_conv(args, np, torch, S, P):
-    """Secondary workloads: the sparse Conv2D configs (cfg3, cfg4), NHWC, one step = one exec of the
-    operator (im2col, SpMM and transpose launches on one stream).  Same JSON shape as the headline."""
-    from oracle import oracle as O
-    from tests.gpu_util import to_dev, upload_weight
+    """The sparse Conv2D configs (cfg3, cfg4), NHWC; one step = one exec of the operator, i.e. every launch
+    the chosen form of the convolution puts on the stream.  Same JSON shape as the SpMM line."""
+    from oracle import oracle as O  # correctness gate and CPU baseline only
     c = P.CONV_CONFIGS[args.config]
     B, H, W, C, F, R, Sx, stride, V, d = [c[k] for k in ("B", "H", "W", "C", "F", "R", "S", "stride", "V", "d")]
     Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
     npix = B * Ho * Wo
     stream = torch.cuda.current_stream()
+    variant = max(args.variant, 0)
 
     def make_op(w, x):
-        f = upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
-        dX = to_dev(torch, x)
+        f = P.upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
+        dX = P.to_dev(torch, x)
         dY = torch.full((B, Ho, Wo, F), float("nan"), dtype=torch.float16, device="cuda")
-        op = S.SpconvBlockwiseOp(max(args.variant, 0))
+        op = S.SpconvBlockwiseOp(variant)
         op.initialize(f, B, H, W, stride, dX.data_ptr(), dY.data_ptr())
         return op, f, dX, dY
 
@@ -270,7 +293,6 @@ def bench_conv(args, np, torch, S, P):
     if not np.array_equal(dYi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
         print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
         sys.exit(1)
-    del opi, fi, dXi, dYi
 
     w = P.make_weight(F, R * Sx * C, V, d, True, 2021, dist=c["w_dist"])
     x = P.make_dense(B * H * W, C, 2021, dist=c["x_dist"]).reshape(B, H, W, C)
@@ -278,50 +300,47 @@ def bench_conv(args, np, torch, S, P):
     nnzb = w["nnzb"]
     eff_flops = 2.0 * nnzb * V * npix
     alg_bytes = nnzb * V * 2 + (nnzb + F // V + 1 + F) * 4 + B * H * W * C * 2 + npix * F * 2
-    for _ in range(args.warmup):
-        op(stream.cuda_stream)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(args.steps):
-        op(stream.cuda_stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / args.steps
+
+    ref_loop_ms = reference_loop(torch, stream, op)
+    ms, wall = timed_region(torch, stream, op, args.steps, args.warmup)
     t = ms * 1e-3
+    int_ms, _ = timed_region(torch, stream, opi, args.steps, args.warmup)
+    del opi, fi, dXi, dYi
+
     cpu = None
     if not args.no_cpu:
-        t0 = time.time()
-        P.conv_oracle(w, R, Sx, C, x, stride)
-        t_all = time.time() - t0
-        cpu = {"value": round(eff_flops / t_all / 1e12, 6), "unit": "TFLOP/s", "cores": O.max_threads(), "kind": "port",
-               "sample": "whole workload, one pass: %.2f s" % t_all}
-    ai = eff_flops / alg_bytes
-    mfma_bound = ai * HBM_PEAK_GBS * 1e9 > MFMA_F16_PEAK_TFLOPS * 1e12
+        X = F // V
+        XS = max(1, X // 8)
+        sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
+                   values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
+        cpu = cpu_baseline(lambda: P.conv_oracle(w, R, Sx, C, x, stride),
+                           lambda: P.conv_oracle(sub, R, Sx, C, x, stride, nthreads=1), eff_flops,
+                           2.0 * int(w["indptr"][XS]) * V * npix, "whole workload (%d panels)" % X,
+                           "the first %d panels" % XS, O.max_threads())
+
     eff_tflops = eff_flops / t / 1e12
-    roof = ({"bound": "mfma", "achieved": round(eff_tflops, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-             "frac": round(eff_tflops / MFMA_F16_PEAK_TFLOPS, 4)} if mfma_bound else
-            {"bound": "hbm", "achieved": round(alg_bytes / t / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-             "frac": round(alg_bytes / t / 1e9 / HBM_PEAK_GBS, 4)})
-    roof.update({"traffic": None, "algorithmic_bytes": alg_bytes, "effective_flops": eff_flops})
+    kernel = S.spconv_variant_name(variant)
+    traffic = measured_traffic(args.config, kernel) if args.traffic is None else round(float(args.traffic))
     print(json.dumps({
         "metric": "effective sparse TFLOP/s + %% fp16 MFMA peak, SpConv2D %s" % args.config,
         "value": round(eff_tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 (fp32 accumulate)",
-        "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter N(0, 0.05), input N(0, 1)",
+        "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter %s(%g), input %s(%g)"
+                % (c["w_dist"] + c["x_dist"]),
         "config": {"workload": "%s: sparse Conv2D NHWC %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
                                "nnzb=%d" % (args.config, B, H, W, C, F, R, Sx, stride, V, d, nnzb),
-                   "kernel": {0: "plane layout + SpMM (tap offsets in the gather) + transpose", 1: "direct",
-                              2: "im2col matrix + SpMM + transpose"}[max(args.variant, 0)]},
+                   "kernel": kernel, "timing": "events around %d back-to-back execs, operands resident" % args.steps},
         "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
-        "reference_timing_loop": {"what": "11 warm-ups + 100 launches from an idle GPU (clock still ramping)",
+        "reference_timing_loop": {"what": "11 warm-ups + 100 execs from an idle GPU (clock still ramping)",
                                   "ms_per_step": round(ref_loop_ms, 6),
                                   "tflops": round(eff_flops / (ref_loop_ms * 1e-3) / 1e12, 1)},
         "integer_valued_operands": {"what": "same mask and shape, values in {-4..4} (the reference's generator)",
                                     "ms_per_step": round(int_ms, 6),
                                     "tflops": round(eff_flops / (int_ms * 1e-3) / 1e12, 1)},
-        "roofline": roof, "cpu_baseline": cpu, "device": S.device_info()}))
+        "dense_equivalent_tflops": round(2.0 * npix * F * R * Sx * C / t / 1e12, 1),
+        "roofline": roofline(eff_flops, alg_bytes, t, traffic), "cpu_baseline": cpu,
+        "wall_s_timed_region": round(wall, 4), "device": S.device_info()}))
 
 
 if __name__ == "__main__":

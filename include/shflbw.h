@@ -104,6 +104,17 @@ int shflbw_weight_set_values(shflbw_weight* w, const uint16_t* values, size_t co
 int shflbw_weight_dump_text(const shflbw_weight* w, char* buf, size_t cap, size_t* needed);
 int shflbw_weight_load_text(shflbw_weight* w, const char* text, size_t len);
 
+/* CPU reference results for a caller's own checks.  Replaces get_host_reference of
+ * blockwise_format.h:268-311 (SpMM: D_ref = alpha * A*B + beta * C, fp32, M x N row-major; C may be
+ * NULL when beta == 0) and of spconv/blockwise_format.h:55-132 (convolution; here over NHWC tensors with
+ * true stride: IFMap[b][hi][wi][c] fp16 bits, OFMap_ref[b][ho][wo][f] fp32, padding R/2, S/2).  Every
+ * element is the fp32 sum in ascending order of the kept vectors, as in the reference.  Host arrays
+ * in, host array out; works on any initialised weight, synced or not. */
+int shflbw_spmm_host_reference(const shflbw_weight* w, int N, const uint16_t* B, float alpha,
+                               const uint16_t* C, float beta, float* D_ref);
+int shflbw_spconv_host_reference(const shflbw_weight* filter, int B, int H, int W, int stride,
+                                 const uint16_t* IFMap, float* OFMap_ref);
+
 int shflbw_weight_get_info(const shflbw_weight* w, shflbw_weight_info* info);
 /* Borrowed pointers to the host arrays (valid until the weight is re-initialised/destroyed). */
 int shflbw_weight_host_arrays(const shflbw_weight* w, const int** indptr, const int** indices,
@@ -226,6 +237,16 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* filter,
 int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* filter,
                                int B, int H, int W, int stride, const void* IFMap, void* OFMap, int variant);
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream);
+/* Forms of the convolution shflbw_spconv_init_variant accepts, and a short name for each. */
+int shflbw_spconv_variant_count(void);
+const char* shflbw_spconv_variant_name(int variant);
+/* Frees the device scratch every shflbw_spconv_init on this filter allocated; states made before
+ * dangle (the reference has no scratch; its states dangle the same way when the filter is
+ * re-initialised, spmm/blockwise_op.h:118-122). */
+int shflbw_weight_release_scratch(shflbw_weight* filter);
+
+/* sizeof the two state structs as this library was compiled, for FFI mirrors to check their layout. */
+void shflbw_abi_sizes(size_t* spmm_state_bytes, size_t* spconv_state_bytes);
 
 /* Library / device facts (for logs): compute units, clock (kHz), LDS bytes per workgroup. */
 int shflbw_device_info(int* compute_units, int* clock_khz, size_t* lds_bytes, char* arch, size_t arch_cap);

@@ -4,7 +4,7 @@ implicit-GEMM sparse Conv2D.  The product is the HIP library behind the C ABI of
 operator interface used by the tests and the benchmark."""
 from . import capi
 from .host import (BlockwiseSpFilter, BlockwiseSpMatrix, SpconvBlockwiseOp, SpmmBlockwiseOp, device_info,
-                   random_mask, spmm_variants)
+                   random_mask, spconv_variant_name, spconv_variants, spmm_variants)
 
 __all__ = ["capi", "BlockwiseSpMatrix", "BlockwiseSpFilter", "SpmmBlockwiseOp", "SpconvBlockwiseOp", "random_mask",
-           "spmm_variants", "device_info"]
+           "spmm_variants", "spconv_variants", "spconv_variant_name", "device_info"]

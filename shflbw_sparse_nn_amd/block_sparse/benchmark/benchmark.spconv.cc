@@ -12,41 +12,21 @@
 #include "block_sparse/cuda_array.h"
 #include "block_sparse/spconv/spconv_library_decl.h"
 #include "block_sparse/spconv/spconv_op.h"
-#include "timing_util.h"
+#include "launch_timing.h"
 
 #define GPU_ARCH 950
 
-static float benchmark(SpconvBlockwiseInitFn_t init_fn, SpconvBlockwiseExecFn_t exec_fn, BlockwiseSpFilter<half>& spfilter,
-                       int B, int Hin, int Win, int stride, half* IFMap, half* OFMap, hipStream_t stream = nullptr,
-                       int warmup = 10, int repeat = 100)
+// one table entry on one problem: mean milliseconds per launch on `stream`, negative when the entry could not run
+static float run_entry(SpconvBlockwiseInitFn_t init_fn, SpconvBlockwiseExecFn_t exec_fn, BlockwiseSpFilter<half>& spfilter,
+                       int B, int Hin, int Win, int stride, half* IFMap, half* OFMap, hipStream_t stream = nullptr)
 {
-    (void)hipDeviceSynchronize();
-    if (hipGetLastError() != hipSuccess) {
-        std::cerr << "return due to previous error. ";
-        return -1;
-    }
-    GpuTimer gpu_timer;
+    if (!launch_timing::device_clean("before the operator was set up")) return -1.f;
     SpconvBlockwiseOpState state = (*init_fn)(spfilter, B, Hin, Win, stride, IFMap, OFMap);
     if (!state.initSuccess) {
-        std::cerr << "return due to unsuccessful initialization. " << std::endl;
-        return -1;
+        std::cerr << "operator set-up failed for this tile name" << std::endl;
+        return -1.f;
     }
-    (*exec_fn)(state, stream);
-    (void)hipDeviceSynchronize();
-    if (!isHipSuccess(hipGetLastError())) {
-        std::cerr << "kernel failed." << std::endl;
-        return -1;
-    }
-    for (int i = 0; i < warmup + repeat; i++) {
-        if (i == warmup) gpu_timer.start();
-        (*exec_fn)(state, stream);
-    }
-    gpu_timer.stop();
-    if (!isHipSuccess(hipGetLastError())) {
-        std::cerr << "kernel failed." << std::endl;
-        return -1;
-    }
-    return gpu_timer.elapsed_msecs() / repeat;
+    return launch_timing::mean_launch_ms([&] { (*exec_fn)(state, stream); }, stream, /* warmup */ 10, /* repeat */ 100);
 }
 
 struct TableEntry {
@@ -74,7 +54,10 @@ int main(int argc, const char** argv)
     CudaRandomArray<half> IFMap;
     CudaZerosArray<half> OFMap;
     IFMap.initialize(a.B * Hin * Win * a.C);
-    OFMap.initialize(a.B * a.H * a.W * F);
+    // the library writes B x Ho x Wo x F; for odd filters that is exactly the H x W of the command line, for an
+    // even R or S the padding R/2 makes it one larger (the reference always writes H x W)
+    const int Ho = (Hin + 2 * (a.R / 2) - a.R) / a.stride + 1, Wo = (Win + 2 * (a.S / 2) - a.S) / a.stride + 1;
+    OFMap.initialize(a.B * Ho * Wo * F);
     IFMap.sync_device();
     OFMap.sync_device();
     if (a.pattern_code != 0) return 0;
@@ -94,7 +77,7 @@ int main(int argc, const char** argv)
         std::cout << GPU_ARCH << " " << spfilter.config_str << " ";
         printf("%d %d %d %d %d %d %d %d %d %d %d %d %d %d ", a.B, a.H, a.W, a.stride, e.t[0], e.t[1], e.t[2], e.t[3],
                e.t[4], e.t[5], e.t[6], e.t[7], e.t[8], e.t[9]);
-        const float dur = benchmark(*e.init, *e.exec, spfilter, a.B, Hin, Win, a.stride, IFMap.device_ptr, OFMap.device_ptr);
+        const float dur = run_entry(*e.init, *e.exec, spfilter, a.B, Hin, Win, a.stride, IFMap.device_ptr, OFMap.device_ptr);
         printf("%f (us) %f (effective tflop/s)\n", dur * 1e3, gflop_count / dur);
         fflush(stdout);
         lines++;

@@ -12,40 +12,21 @@
 #include "block_sparse/cuda_array.h"
 #include "block_sparse/spmm/spmm_library_decl.h"
 #include "block_sparse/spmm/spmm_op.h"
-#include "timing_util.h"
+#include "launch_timing.h"
 
 #define GPU_ARCH 950 // gfx950; the reference prints its compute capability in this column
 
-static float benchmark(SpmmBlockwiseInitFn_t init_fn, SpmmBlockwiseExecFn_t exec_fn, BlockwiseSpMatrix<half>& spmat, int N,
-                       half* B, half* D, hipStream_t stream = nullptr, int warmup = 10, int repeat = 100)
+// one table entry on one problem: mean milliseconds per launch on `stream`, negative when the entry could not run
+static float run_entry(SpmmBlockwiseInitFn_t init_fn, SpmmBlockwiseExecFn_t exec_fn, BlockwiseSpMatrix<half>& spmat, int N,
+                       half* B, half* D, hipStream_t stream = nullptr)
 {
-    (void)hipDeviceSynchronize();
-    if (hipGetLastError() != hipSuccess) {
-        std::cerr << "return due to previous error. ";
-        return -1;
-    }
-    GpuTimer gpu_timer;
+    if (!launch_timing::device_clean("before the operator was set up")) return -1.f;
     SpmmBlockwiseOpState state = (*init_fn)(spmat, N, B, D);
     if (!state.initSuccess) {
-        std::cerr << "return due to unsuccessful initialization. " << std::endl;
-        return -1;
+        std::cerr << "operator set-up failed for this tile name" << std::endl;
+        return -1.f;
     }
-    (*exec_fn)(state, stream);
-    (void)hipDeviceSynchronize();
-    if (!isHipSuccess(hipGetLastError())) {
-        std::cerr << "kernel failed." << std::endl;
-        return -1;
-    }
-    for (int i = 0; i < warmup + repeat; i++) {
-        if (i == warmup) gpu_timer.start();
-        (*exec_fn)(state, stream);
-    }
-    gpu_timer.stop();
-    if (!isHipSuccess(hipGetLastError())) {
-        std::cerr << "kernel failed." << std::endl;
-        return -1;
-    }
-    return gpu_timer.elapsed_msecs() / repeat;
+    return launch_timing::mean_launch_ms([&] { (*exec_fn)(state, stream); }, stream, /* warmup */ 10, /* repeat */ 100);
 }
 
 struct TableEntry {
@@ -99,7 +80,7 @@ int main(int argc, const char** argv)
         std::cout << GPU_ARCH << " " << spmat.config_str << " ";
         printf("%d %d %d %d %d %d %d %d %d %d %d ", n, e.t[0], e.t[1], e.t[2], e.t[3], e.t[4], e.t[5], e.t[6], e.t[7],
                e.t[8], e.t[9]);
-        const float dur = benchmark(*e.init, *e.exec, spmat, n, B.device_ptr, D.device_ptr);
+        const float dur = run_entry(*e.init, *e.exec, spmat, n, B.device_ptr, D.device_ptr);
         printf("%f (us) %f (effective tflop/s)\n", dur * 1e3, gflop_count / dur);
         fflush(stdout);
         lines++;

@@ -25,4 +25,27 @@ struct BlockwiseSpFilter : public BlockwiseSpMatrix<T> {
         this->filter_R_ = R_, this->filter_S_ = S_, this->filter_C_ = C_;
         this->pull_host_arrays();
     }
+
+    template <typename U>
+    friend void get_host_reference(BlockwiseSpFilter<U>& spfilter, const int B, const int H, const int W,
+                                   const int stride, const std::vector<U>& IFMap, std::vector<float>& OFMap_ref,
+                                   LayoutFilter layout_filter);
 };
+
+// The convolution on the CPU, fp32 (spconv/blockwise_format.h:55-132), over this library's tensors: NHWC,
+// H and W are the input extents, padding R/2 and S/2, output [B][Ho][Wo][F] with
+// Ho = (H + 2*(R/2) - R)/stride + 1.  Only filter_channel_first filters exist here.
+template <typename T>
+void get_host_reference(BlockwiseSpFilter<T>& spfilter, const int B, const int H, const int W, const int stride,
+                        const std::vector<T>& IFMap, std::vector<float>& OFMap_ref,
+                        LayoutFilter layout_filter = filter_channel_first)
+{
+    assert(layout_filter == filter_channel_first);
+    (void)layout_filter;
+    spfilter.push_host_arrays();
+    const int Ho = (H + 2 * (spfilter.R / 2) - spfilter.R) / stride + 1;
+    const int Wo = (W + 2 * (spfilter.S / 2) - spfilter.S) / stride + 1;
+    OFMap_ref.resize(static_cast<size_t>(B) * Ho * Wo * spfilter.F);
+    SHFLBW_CHECK(shflbw_spconv_host_reference(spfilter.handle(), B, H, W, stride,
+                                              reinterpret_cast<const uint16_t*>(IFMap.data()), OFMap_ref.data()));
+}

@@ -72,6 +72,8 @@ struct BlockwiseSpMatrix {
         pull_host_arrays();
     }
 
+    // read-only as in the reference (blockwise_format.h:125-149): handing over vectors the library already
+    // holds changes nothing, so a synced weight stays synced and its operator states stay valid
     void dump(std::ostream& out)
     {
         push_host_arrays();
@@ -140,6 +142,28 @@ protected:
                                        reinterpret_cast<const uint16_t*>(values.data()),
                                        row_permute ? row_permute_ids.data() : nullptr, filter_R_, filter_S_,
                                        filter_C_));
+        // edited vectors drop the device image, as a new init_random does in the reference (:118-122)
+        shflbw_weight_info info;
+        SHFLBW_CHECK(shflbw_weight_get_info(handle_, &info));
+        device_synced = info.device_synced != 0;
     }
 
+    template <typename U>
+    friend void get_host_reference(BlockwiseSpMatrix<U>& spmat, const int N, const std::vector<U>& B, float alpha,
+                                   const std::vector<U>& C, float beta, std::vector<float>& D_ref);
+
 };
+
+// D_ref = alpha * A*B + beta * C on the CPU, fp32, M x N row-major (blockwise_format.h:268-311): the check
+// the reference's examples run after the GPU launch.  Computed by the library's host code from the public
+// vectors of `spmat`.
+template <typename T>
+void get_host_reference(BlockwiseSpMatrix<T>& spmat, const int N, const std::vector<T>& B, float alpha,
+                        const std::vector<T>& C, float beta, std::vector<float>& D_ref)
+{
+    spmat.push_host_arrays();
+    D_ref.resize(static_cast<size_t>(spmat.nrow) * N);
+    SHFLBW_CHECK(shflbw_spmm_host_reference(spmat.handle(), N, reinterpret_cast<const uint16_t*>(B.data()), alpha,
+                                            C.empty() ? nullptr : reinterpret_cast<const uint16_t*>(C.data()),
+                                            C.empty() ? 0.f : beta, D_ref.data()));
+}

@@ -23,7 +23,9 @@ EXPORTS = [
     "shflbw_spmm_init", "shflbw_spmm_init_variant", "shflbw_spmm_exec",
     "shflbw_spmm_variant_count", "shflbw_spmm_variant_name",
     "shflbw_spconv_init", "shflbw_spconv_init_variant", "shflbw_spconv_exec",
-    "shflbw_device_info",
+    "shflbw_spconv_variant_count", "shflbw_spconv_variant_name", "shflbw_weight_release_scratch",
+    "shflbw_spmm_host_reference", "shflbw_spconv_host_reference",
+    "shflbw_abi_sizes", "shflbw_device_info",
 ]
 
 OK = 0
@@ -52,7 +54,7 @@ class SpmmState(C.Structure):
     _fields_ = [("shared_mem_size", C.c_size_t), ("grid_dim", C.c_uint * 3), ("block_dim", C.c_uint * 3),
                 ("init_success", C.c_int), ("variant", C.c_int), ("args", _SpmmArgs),
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("packed_indices_pm", C.c_void_p),
-                ("panel_ptr", C.c_void_p), ("brow", C.c_int)]
+                ("panel_ptr", C.c_void_p), ("brow", C.c_int), ("ldb_bytes", C.c_int)]
 
 
 class _SpconvArgs(C.Structure):
@@ -117,7 +119,21 @@ def load():
     lib.shflbw_spconv_init.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp]
     lib.shflbw_spconv_init_variant.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp, ci]
     lib.shflbw_spconv_exec.argtypes = [C.POINTER(SpconvState), vp]
+    lib.shflbw_spconv_variant_count.argtypes = []
+    lib.shflbw_spconv_variant_name.restype = C.c_char_p
+    lib.shflbw_spconv_variant_name.argtypes = [ci]
+    lib.shflbw_weight_release_scratch.argtypes = [vp]
+    lib.shflbw_spmm_host_reference.argtypes = [vp, ci, vp, cf, vp, cf, vp]
+    lib.shflbw_spconv_host_reference.argtypes = [vp, ci, ci, ci, ci, vp, vp]
+    lib.shflbw_abi_sizes.restype = None
+    lib.shflbw_abi_sizes.argtypes = [C.POINTER(sz), C.POINTER(sz)]
     lib.shflbw_device_info.argtypes = [ip, ip, C.POINTER(sz), C.c_char_p, sz]
+    # the ctypes mirrors above must have the layout the library was compiled with
+    a, b = sz(0), sz(0)
+    lib.shflbw_abi_sizes(C.byref(a), C.byref(b))
+    if (a.value, b.value) != (C.sizeof(SpmmState), C.sizeof(SpconvState)):
+        raise RuntimeError("state struct layout mismatch: library %d/%d bytes, ctypes mirror %d/%d"
+                           % (a.value, b.value, C.sizeof(SpmmState), C.sizeof(SpconvState)))
     _lib = lib
     return lib
 

@@ -6,6 +6,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "shflbw.h"
@@ -106,6 +107,9 @@ static const SpconvVariant* find_spconv_variant(int brow, int variant, int* n_fo
     return hit;
 }
 
+// the persistent role-split variants ("ws..." names) form gather addresses from 32-bit byte offsets
+static bool spmm_variant_offsets32(const SpmmVariant* v) { return v && v->name[0] == 'w'; }
+
 // Tile choice when the caller does not force one: the table lists the preferred (persistent, 512 columns
 // wide) variant of every block size first.  When its tiles would occupy at most half of the compute units,
 // the role-split variant with 256-column tiles is taken instead (twice the tiles; measured 15-25 % faster
@@ -176,10 +180,27 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
         return SHFLBW_ERR_INVALID;
     }
     const int X = w->nrow / w->brow;
-    if (variant < 0) variant = auto_spmm_variant(w->brow, X, N);
+    // the role-split kernels address the rows of B with 32-bit byte offsets
+    const bool wide_b = (unsigned long long)w->ncol * (unsigned long long)N * 2ull + (unsigned long long)N * 2ull > 0xffffffffull;
+    if (variant < 0) {
+        variant = auto_spmm_variant(w->brow, X, N);
+        if (wide_b) { // first variant of this block size with 64-bit addressing
+            int n = 0;
+            find_spmm_variant(w->brow, 0, &n);
+            for (int i = 0; i < n; i++)
+                if (!spmm_variant_offsets32(find_spmm_variant(w->brow, i, nullptr))) {
+                    variant = i;
+                    break;
+                }
+        }
+    }
     const SpmmVariant* v = find_spmm_variant(w->brow, variant, nullptr);
     if (!v) {
         set_error("spmm_init: no tile variant %d for block size %d", variant, w->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (wide_b && spmm_variant_offsets32(v)) {
+        set_error("spmm_init: B (%d x %d fp16) exceeds the 4 GiB the tile variant %s can address", w->ncol, N, v->name);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     SHFLBW_HIP_TRY(v->prepare());
@@ -304,7 +325,7 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         set_error("spconv_init: empty output (%d x %d)", Ho, Wo);
         return SHFLBW_ERR_SHAPE;
     }
-    if (variant < 0 || variant > 2) {
+    if (variant < 0 || variant >= shflbw_spconv_variant_count()) {
         set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = im2col form)", variant);
         return SHFLBW_ERR_INVALID;
     }
@@ -312,6 +333,10 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     if (variant == 1) {
         if (!v) {
             set_error("spconv_init: no direct kernel for block size %d", f->brow);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        if ((unsigned long long)B * H * W * f->C > 0x7fffffffull) {
+            set_error("spconv_init: input of %d x %d x %d x %d values exceeds the 2^31 the direct kernel can index", B, H, W, f->C);
             return SHFLBW_ERR_UNSUPPORTED;
         }
         SHFLBW_HIP_TRY(v->prepare());
@@ -342,17 +367,20 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     state->brow = f->brow;
     state->variant = variant;
     const long npix = (long)B * Ho * Wo;
-    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is not part of the weight's value
+    // The scratch cache is bookkeeping of the handle, not part of the weight's value; it is the one member an
+    // init call changes, under its lock.
+    shflbw_weight* fw = const_cast<shflbw_weight*>(f);
+    std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
     const int key[5] = {variant, B, H, W, stride};
     auto cached_scratch = [&](size_t bytes, bool* fresh) -> void* {
         for (auto& sc : fw->conv_scratch)
-            if (sc.bytes == bytes && memcmp(sc.key, key, sizeof(key)) == 0) {
+            if (sc.bytes == bytes && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap) {
                 *fresh = false;
                 return sc.ptr;
             }
         void* ptr = nullptr;
         if (hipMalloc(&ptr, bytes) != hipSuccess) return nullptr;
-        shflbw_weight::Scratch sc{bytes, ptr, {key[0], key[1], key[2], key[3], key[4]}};
+        shflbw_weight::Scratch sc{bytes, ptr, {key[0], key[1], key[2], key[3], key[4]}, IFMap, OFMap};
         fw->conv_scratch.push_back(sc);
         *fresh = true;
         return ptr;
@@ -528,6 +556,35 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         return SHFLBW_ERR_HIP;
     }
     return SHFLBW_OK;
+}
+
+static const char* const g_spconv_forms[] = {
+    "planes+spmm+transpose",  // 0: NHWC -> channel-major planes, SpMM gather with tap offsets, transpose to NHWC
+    "direct",                 // 1: one kernel, im2col gather from NHWC in the tile loads
+    "im2col+spmm+transpose",  // 2: explicit im2col matrix
+};
+
+int shflbw_spconv_variant_count(void) { return (int)(sizeof(g_spconv_forms) / sizeof(g_spconv_forms[0])); }
+
+const char* shflbw_spconv_variant_name(int variant)
+{
+    return variant >= 0 && variant < shflbw_spconv_variant_count() ? g_spconv_forms[variant] : "";
+}
+
+int shflbw_weight_release_scratch(shflbw_weight* w)
+{
+    if (!w) return SHFLBW_ERR_INVALID;
+    std::lock_guard<std::mutex> guard(w->scratch_lock);
+    for (auto& sc : w->conv_scratch)
+        if (sc.ptr) (void)hipFree(sc.ptr);
+    w->conv_scratch.clear();
+    return SHFLBW_OK;
+}
+
+void shflbw_abi_sizes(size_t* spmm_state_bytes, size_t* spconv_state_bytes)
+{
+    if (spmm_state_bytes) *spmm_state_bytes = sizeof(shflbw_spmm_state);
+    if (spconv_state_bytes) *spconv_state_bytes = sizeof(shflbw_spconv_state);
 }
 
 int shflbw_device_info(int* compute_units, int* clock_khz, size_t* lds_bytes, char* arch, size_t arch_cap)

@@ -416,6 +416,15 @@ int shflbw_weight_set(shflbw_weight* w, int nrow, int ncol, int brow, int bcol, 
         return SHFLBW_ERR_SHAPE;
     }
     const int X = nrow / brow;
+    // Arrays equal to what the weight already holds change nothing: the device image, the states made from it,
+    // the seed and the config string stay valid (the veneer hands its public vectors over before every dump
+    // and sync, and the reference's dump is read-only, blockwise_format.h:125-149).
+    if (w->initialized && w->nrow == nrow && w->ncol == ncol && w->brow == brow && w->bcol == bcol &&
+        w->nnzb == nnzb && w->row_permute == (row_permute_ids != nullptr) && w->R == R && w->S == S && w->C == C &&
+        std::equal(indptr, indptr + X + 1, w->indptr.begin()) && std::equal(indices, indices + nnzb, w->indices.begin()) &&
+        std::equal(values, values + (size_t)nnzb * brow * bcol, w->values.begin()) &&
+        (!row_permute_ids || std::equal(row_permute_ids, row_permute_ids + nrow, w->row_permute_ids.begin())))
+        return SHFLBW_OK;
     w->nrow = nrow;
     w->ncol = ncol;
     w->brow = brow;

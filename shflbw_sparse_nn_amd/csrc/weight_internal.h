@@ -2,6 +2,7 @@
 // Host side of the Shfl-BW format: reference block_sparse/spmm/blockwise_format.h:13-68.
 #pragma once
 #include <cstdint>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -40,16 +41,20 @@ struct shflbw_weight {
     void* d_packed_indices_pm = nullptr;
     void* d_packed_values = nullptr;
 
-    // device scratch of the multi-launch forms of the convolution (layout-transformed input, the
-    // filter-major result and, for the plane form, the kept-column ids rewritten as plane offsets),
-    // one allocation per distinct problem geometry, handed out by shflbw_spconv_init and kept until
-    // the weight is re-initialised or destroyed
+    // Device scratch of the convolution (layout-transformed input, filter-major result, the kept-column ids
+    // rewritten as plane offsets, synchronisation words): one allocation per distinct (form, geometry, input
+    // tensor, output tensor), handed out by shflbw_spconv_init under `scratch_lock` and kept until the weight
+    // is re-initialised or destroyed.  States over different tensors therefore never share scratch; two
+    // states with equal key are the same computation.
     struct Scratch {
         size_t bytes;
         void* ptr;
         int key[5]; // variant, B, H, W, stride
+        const void* in;
+        const void* out;
     };
     std::vector<Scratch> conv_scratch;
+    std::mutex scratch_lock;
 };
 
 namespace shflbw {

@@ -135,6 +135,18 @@ class BlockwiseSpMatrix:
         capi.check(self._lib.shflbw_weight_meta_host(self._h, C.byref(p), C.byref(n)))
         return _np_from(p.value, n.value, np.int32)
 
+    def host_reference(self, N, B, alpha=1.0, Cmat=None, beta=0.0):
+        """get_host_reference (blockwise_format.h:268-311) computed by the library's host code: fp32 M x N."""
+        B = np.ascontiguousarray(B, dtype=np.float16)
+        Cm = None if Cmat is None else np.ascontiguousarray(Cmat, dtype=np.float16)
+        out = np.empty((self.nrow, N), dtype=np.float32)
+        capi.check(self._lib.shflbw_spmm_host_reference(self._h, N, B.ctypes.data, alpha,
+                                                        None if Cm is None else Cm.ctypes.data, beta, out.ctypes.data))
+        return out
+
+    def release_scratch(self):
+        capi.check(self._lib.shflbw_weight_release_scratch(self._h))
+
     @property
     def device_ref(self):
         r = capi.DeviceRef()
@@ -148,6 +160,18 @@ class BlockwiseSpFilter(BlockwiseSpMatrix):
     def init_random(self, F, R, S, Cc, brow, bcol, expected_density, filter_permute, seed):
         capi.check(self._lib.shflbw_filter_init_random(self._h, F, R, S, Cc, brow, bcol, expected_density,
                                                       int(bool(filter_permute)), seed))
+
+    def host_reference(self, x_nhwc, stride):
+        """get_host_reference of the convolution (spconv/blockwise_format.h:55-132) over NHWC tensors: fp32
+        [B][Ho][Wo][F]."""
+        x = np.ascontiguousarray(x_nhwc, dtype=np.float16)
+        Bn, H, W, _ = x.shape
+        i = self.info
+        Ho = (H + 2 * (i.R // 2) - i.R) // stride + 1
+        Wo = (W + 2 * (i.S // 2) - i.S) // stride + 1
+        out = np.empty((Bn, Ho, Wo, i.F), dtype=np.float32)
+        capi.check(self._lib.shflbw_spconv_host_reference(self._h, Bn, H, W, stride, x.ctypes.data, out.ctypes.data))
+        return out
 
 
 class SpmmBlockwiseOp:
@@ -173,7 +197,7 @@ class SpmmBlockwiseOp:
 
 class SpconvBlockwiseOp:
     """initialize(spfilter, B, H, W, stride, IFMap, OFMap); NHWC tensors, H and W are input extents.
-    variant 0 (default): im2col + SpMM + transpose on the stream; variant 1: one direct kernel."""
+    `variant` selects the form of the convolution (spconv_variants() names them); 0 is the library's default."""
 
     def __init__(self, variant=0):
         self._lib = capi.load()
@@ -197,6 +221,15 @@ class SpconvBlockwiseOp:
 def spmm_variants(brow):
     lib = capi.load()
     return [lib.shflbw_spmm_variant_name(brow, v).decode() for v in range(lib.shflbw_spmm_variant_count(brow))]
+
+
+def spconv_variants():
+    lib = capi.load()
+    return [lib.shflbw_spconv_variant_name(v).decode() for v in range(lib.shflbw_spconv_variant_count())]
+
+
+def spconv_variant_name(variant):
+    return capi.load().shflbw_spconv_variant_name(variant).decode()
 
 
 def device_info():

@@ -20,7 +20,7 @@ int oracle_spconv_reference_nhwc(int F, int R, int S, int C, int brow, const int
 }
 
 template <typename T>
-void get_host_reference(BlockwiseSpMatrix<T>& spmat, int N, const std::vector<T>& B, float alpha,
+void oracle_reference(BlockwiseSpMatrix<T>& spmat, int N, const std::vector<T>& B, float alpha,
                         const std::vector<T>& C, float beta, std::vector<float>& D_ref)
 {
     D_ref.assign(static_cast<size_t>(spmat.nrow) * N, 0.f);
@@ -38,7 +38,7 @@ void get_host_reference(BlockwiseSpMatrix<T>& spmat, int N, const std::vector<T>
 
 // NHWC feature maps, H and W are the input extents, padding R/2 and S/2
 template <typename T>
-void get_host_reference(BlockwiseSpFilter<T>& f, int B, int H, int W, int stride, const std::vector<T>& IFMap,
+void oracle_reference(BlockwiseSpFilter<T>& f, int B, int H, int W, int stride, const std::vector<T>& IFMap,
                         std::vector<float>& OFMap_ref)
 {
     const int Ho = (H + 2 * (f.R / 2) - f.R) / stride + 1, Wo = (W + 2 * (f.S / 2) - f.S) / stride + 1;

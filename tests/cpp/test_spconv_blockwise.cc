@@ -8,7 +8,7 @@
 #include "block_sparse/cuda_array.h"
 #include "block_sparse/spconv/spconv_library_decl.h"
 #include "block_sparse/spconv/spconv_op.h"
-#include "host_reference.h"
+#include "oracle_reference.h"
 
 struct TableEntry {
     const char* name;
@@ -63,8 +63,8 @@ static int test_block_size(int block_sz, int n, int h, int w, int c, int f, int 
     OFMap.initialize(n * h * w * f);
 
     std::vector<float> ref_plain, ref_permuted;
-    get_host_reference<half>(plain, n, h_in, w_in, stride, IFMap.host_array, ref_plain);
-    get_host_reference<half>(permuted, n, h_in, w_in, stride, IFMap.host_array, ref_permuted);
+    oracle_reference<half>(plain, n, h_in, w_in, stride, IFMap.host_array, ref_plain);
+    oracle_reference<half>(permuted, n, h_in, w_in, stride, IFMap.host_array, ref_permuted);
     if (ref_plain.size() != static_cast<size_t>(OFMap.size)) {
         std::cerr << "output extent mismatch\n";
         return 1;

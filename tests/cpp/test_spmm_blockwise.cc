@@ -9,7 +9,7 @@
 #include "block_sparse/cuda_array.h"
 #include "block_sparse/spmm/spmm_library_decl.h"
 #include "block_sparse/spmm/spmm_op.h"
-#include "host_reference.h"
+#include "oracle_reference.h"
 
 struct TableEntry {
     const char* name;
@@ -62,8 +62,8 @@ static int test_block_size(int block_sz, int m, int n, int k, float density, uns
     D.initialize(m * n);
 
     std::vector<float> ref_plain, ref_permuted;
-    get_host_reference<half>(plain, n, B.host_array, 1.0f, C.host_array, 0.0f, ref_plain);
-    get_host_reference<half>(permuted, n, B.host_array, 1.0f, C.host_array, 0.0f, ref_permuted);
+    oracle_reference<half>(plain, n, B.host_array, 1.0f, C.host_array, 0.0f, ref_plain);
+    oracle_reference<half>(permuted, n, B.host_array, 1.0f, C.host_array, 0.0f, ref_permuted);
 
     for (const TableEntry& e : table) {
         if (e.block_sz != block_sz) continue;
@@ -79,7 +79,7 @@ static int test_block_size(int block_sz, int m, int n, int k, float density, uns
         CudaOnesArray<half> ones;
         ones.initialize(m * n);
         std::vector<float> ref;
-        get_host_reference<half>(permuted, n, B.host_array, 1.0f, ones.host_array, 1.0f, ref);
+        oracle_reference<half>(permuted, n, B.host_array, 1.0f, ones.host_array, 1.0f, ref);
         bool ok = false;
         auto run = [&](auto& op) {
             op.initialize(permuted, n, B.device_ptr, ones.device_ptr, D.device_ptr);

@@ -7,8 +7,8 @@ import pytest
 
 import shflbw_sparse_nn_amd as S
 from oracle import oracle as O
-from tests import problems as P
-from tests.gpu_util import to_dev, upload_weight
+import workloads as P
+from workloads import to_dev, upload_weight
 
 pytestmark = pytest.mark.gpu
 

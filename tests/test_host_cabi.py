@@ -161,3 +161,55 @@ def test_static_archive_holds_the_operator_tables():
         for kind in ("SpmmBlockwise", "SpconvBlockwise"):
             for fn in ("Init", "Exec"):
                 assert "%s_%s_%sFn" % (kind, tag, fn) in syms, (kind, tag, fn)
+
+
+def test_state_struct_layout_matches_the_library():
+    lib = capi.load()  # load() itself raises on a mismatch; spell the figures out here
+    a, b = C.c_size_t(0), C.c_size_t(0)
+    lib.shflbw_abi_sizes(C.byref(a), C.byref(b))
+    assert (a.value, b.value) == (C.sizeof(capi.SpmmState), C.sizeof(capi.SpconvState))
+    assert capi.SpmmState.ldb_bytes.offset == capi.SpmmState.brow.offset + 4
+
+
+def test_spconv_forms_are_named():
+    names = S.spconv_variants()
+    assert len(names) >= 3 and len(set(names)) == len(names) and all(names)
+    assert S.spconv_variant_name(len(names)) == ""
+
+
+def test_set_with_equal_arrays_is_a_no_op():
+    """dump() of the C++ veneer hands its public vectors back to the library first; when nothing changed
+    the weight must keep its seed and config string (a changed one would mean the set went through
+    and, on a synced weight, dropped the device image)."""
+    m = S.BlockwiseSpMatrix()
+    m.init_random(256, 128, 32, 1, 0.25, True, 99)
+    cfg, seed = m.config_str, m.seed
+    m.set(256, 128, 32, 1, m.indptr, m.indices, m.values, m.row_permute_ids)
+    assert (m.config_str, m.seed) == (cfg, seed) and seed == 99
+    v = m.values.copy()
+    v[0] = v[0] + 1
+    m.set(256, 128, 32, 1, m.indptr, m.indices, v, m.row_permute_ids)
+    assert m.seed == 0  # a real change goes through
+
+
+@pytest.mark.parametrize("V,permute", [(16, True), (32, False), (64, True)])
+def test_library_spmm_host_reference_equals_the_oracle(V, permute):
+    import workloads as P
+    w = P.make_weight(128, 96, V, 0.3, permute, 5, dist=("normal", 1.0))
+    B = P.make_dense(96, 40, 5, dist=("uniform", 1.0))
+    Cm = P.make_dense(128, 40, 6, dist=("uniform", 1.0))
+    m = S.BlockwiseSpMatrix()
+    m.set(w["nrow"], w["ncol"], V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"])
+    np.testing.assert_array_equal(m.host_reference(40, B), P.spmm_oracle(w, B))
+    np.testing.assert_array_equal(m.host_reference(40, B, 0.5, Cm, -2.0), P.spmm_oracle(w, B, Cm, 0.5, -2.0))
+
+
+@pytest.mark.parametrize("stride,R,Sx", [(1, 3, 3), (2, 3, 3), (2, 5, 1), (1, 1, 1)])
+def test_library_spconv_host_reference_equals_the_oracle(stride, R, Sx):
+    import workloads as P
+    Cc, F, V = 16, 64, 32
+    w = P.make_weight(F, R * Sx * Cc, V, 0.3, True, 11, dist=("normal", 1.0))
+    x = np.random.default_rng(3).standard_normal((2, 9, 7, Cc)).astype(np.float16)
+    f = S.BlockwiseSpFilter()
+    f.set(F, R * Sx * Cc, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"], R, Sx, Cc)
+    np.testing.assert_array_equal(f.host_reference(x, stride), P.conv_oracle(w, R, Sx, Cc, x, stride))

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
-from tests import problems as P
+import workloads as P
 
 # example/spmatrix_dump_load.md:22-41 (plain) and :66-91 (with row permutation 0 3 1 2)
 DOC_PLAIN = """4\n4\n2\n2\n2\n0\n0 1 2\n0 1\n1 2 1 2 3 1 1 2\n"""

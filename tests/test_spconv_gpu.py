@@ -6,8 +6,8 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
-from tests import problems as P
-from tests.gpu_util import float_error_report, run_spconv
+import workloads as P
+from workloads import float_error_report, run_spconv
 
 pytestmark = pytest.mark.gpu
 

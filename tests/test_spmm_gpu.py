@@ -10,8 +10,8 @@ import pytest
 
 import shflbw_sparse_nn_amd as S
 from oracle import oracle as O
-from tests import problems as P
-from tests.gpu_util import float_error_report, run_spmm
+import workloads as P
+from workloads import float_error_report, run_spmm
 
 pytestmark = pytest.mark.gpu
 
