@@ -237,6 +237,19 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* filter,
 int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* filter,
                                int B, int H, int W, int stride, const void* IFMap, void* OFMap, int variant);
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream);
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  One complete convolution in the plane
+ * form, the same launches as shflbw_spconv_init + shflbw_spconv_exec, with all scratch (the planes, the
+ * filter-major result, the rewritten ids, which a small kernel computes on the device) in a fixed device
+ * array inside the library: SHFLBW_STATIC_SCRATCH_BYTES on every GPU the library runs on, held until the
+ * process ends.  Calls no hipMalloc / hipFree and copies nothing from the host; launches on `stream` only.
+ * A problem whose scratch exceeds the array is refused with SHFLBW_ERR_CAPACITY (the message names both
+ * sizes).  All calls on one GPU share the array: calls that overlap in time on one GPU race, also on
+ * different streams; calls in stream order are safe, nothing of an earlier call is relied on. */
+#define SHFLBW_STATIC_SCRATCH_BYTES (40u * 1024u * 1024u)
+int shflbw_spconv_exec_static(const shflbw_weight* filter, int B, int H, int W, int stride,
+                              const void* IFMap, void* OFMap, void* stream);
+
 /* Forms of the convolution shflbw_spconv_init_variant accepts, and a short name for each. */
 int shflbw_spconv_variant_count(void);
 const char* shflbw_spconv_variant_name(int variant);

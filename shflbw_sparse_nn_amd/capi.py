@@ -23,6 +23,7 @@ EXPORTS = [
     "shflbw_spmm_init", "shflbw_spmm_init_variant", "shflbw_spmm_exec",
     "shflbw_spmm_variant_count", "shflbw_spmm_variant_name",
     "shflbw_spconv_init", "shflbw_spconv_init_variant", "shflbw_spconv_exec",
+    "shflbw_spconv_exec_static",
     "shflbw_spconv_variant_count", "shflbw_spconv_variant_name", "shflbw_weight_release_scratch",
     "shflbw_spmm_host_reference", "shflbw_spconv_host_reference",
     "shflbw_abi_sizes", "shflbw_device_info",
@@ -30,6 +31,7 @@ EXPORTS = [
 
 OK = 0
 ERR_INVALID, ERR_SHAPE, ERR_STATE, ERR_HIP, ERR_UNSUPPORTED, ERR_FORMAT, ERR_CAPACITY = range(1, 8)
+STATIC_SCRATCH_BYTES = 40 * 1024 * 1024  # SHFLBW_STATIC_SCRATCH_BYTES
 
 
 class WeightInfo(C.Structure):
@@ -119,6 +121,7 @@ def load():
     lib.shflbw_spconv_init.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp]
     lib.shflbw_spconv_init_variant.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp, ci]
     lib.shflbw_spconv_exec.argtypes = [C.POINTER(SpconvState), vp]
+    lib.shflbw_spconv_exec_static.argtypes = [vp, ci, ci, ci, ci, vp, vp, vp]
     lib.shflbw_spconv_variant_count.argtypes = []
     lib.shflbw_spconv_variant_name.restype = C.c_char_p
     lib.shflbw_spconv_variant_name.argtypes = [ci]

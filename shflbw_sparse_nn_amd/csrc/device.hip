@@ -131,6 +131,44 @@ static int auto_spmm_variant(int brow, int X, int N)
     return 0;
 }
 
+// Geometry of the plane form of a convolution and the layout of its device scratch.
+struct PlaneForm {
+    int PH, PW;     // rows and (padded to 8) columns of one phase plane
+    int copies;     // 2 when some tap offset is odd (a second copy moved by one value keeps gathers aligned)
+    long np;        // plane positions = columns of the SpMM in the middle
+    long pitch;     // values per channel row of the plane tensor
+    long rows;      // channel rows: copies * stride^2 * C
+    size_t slots;   // padded kept-vector slots of the filter
+    size_t planes_bytes, dm_bytes, ids_bytes; // scratch = planes | result_fm | ids | ids_pm
+    size_t total_bytes() const { return planes_bytes + dm_bytes + 2 * ids_bytes; }
+};
+
+static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int stride, PlaneForm* g)
+{
+    const int s = stride, ph = f->R / 2, pw = f->S / 2;
+    g->PH = (H + 2 * ph + s - 1) / s;
+    g->PW = ((W + 2 * pw + s - 1) / s + 7) / 8 * 8;
+    g->np = (long)B * g->PH * g->PW;
+    const long max_shift = (long)((f->R - 1) / s) * g->PW + (f->S - 1) / s; // largest tap offset
+    g->pitch = (g->np + max_shift + 8 + 63) / 64 * 64;
+    g->copies = (f->S - 1) / s >= 1 ? 2 : 1;
+    if (g->copies * s * s > 32) {
+        set_error("spconv: stride %d has too many phase planes for the plane form", s);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    g->rows = (long)g->copies * s * s * f->C;
+    if (g->np > 0x7fffffffL || (unsigned long long)g->rows * (unsigned long long)g->pitch * 2ull > 0xffffffffull) {
+        set_error("spconv: problem too large for the plane form (%ld rows of %ld positions)", g->rows, g->pitch);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
+    g->slots = f->packed_indices.size();
+    g->planes_bytes = up256((size_t)g->rows * g->pitch * 2);
+    g->dm_bytes = up256((size_t)f->F * g->np * 2);
+    g->ids_bytes = up256(g->slots * sizeof(int) + 64);
+    return SHFLBW_OK;
+}
+
 } // namespace shflbw
 
 using namespace shflbw;
@@ -286,8 +324,9 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B
     return shflbw_spconv_init_variant(state, f, B, H, W, stride, IFMap, OFMap, 0);
 }
 
-int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                               const void* IFMap, void* OFMap, int variant)
+// Argument checks of a convolution and every field of the state that does not depend on device scratch.
+static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                             const void* IFMap, void* OFMap, int variant)
 {
     if (!state) return SHFLBW_ERR_INVALID;
     memset(state, 0, sizeof(*state));
@@ -366,6 +405,43 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     state->panel_ptr = (const int*)f->d_group_ptr;
     state->brow = f->brow;
     state->variant = variant;
+    return SHFLBW_OK;
+}
+
+// Points a state of the plane form at its scratch (planes | result_fm | ids | ids_pm, laid out by `g`) and sets
+// up the SpMM launch in the middle.  The ids must be in the scratch when the state is executed.
+static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, const PlaneForm& g, char* scratch)
+{
+    state->planes = scratch;
+    state->result_fm = scratch + g.planes_bytes;
+    state->np = (int)g.np;
+    state->plane_rows = g.PH;
+    state->plane_cols = g.PW;
+    state->plane_pitch = (int)g.pitch;
+    state->plane_copies = g.copies;
+    int rc = shflbw_spmm_init(&state->spmm, f, (int)g.np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
+    if (rc != SHFLBW_OK) return rc;
+    // the gather walks the planes: ids are element offsets, one id apart is one value apart
+    state->spmm.packed_indices = (const int*)(scratch + g.planes_bytes + g.dm_bytes);
+    state->spmm.packed_indices_pm = (const int*)(scratch + g.planes_bytes + g.dm_bytes + g.ids_bytes);
+    state->spmm.ldb_bytes = 2;
+    state->spmm.args.K = (int)(g.rows * g.pitch); // extent of the id space
+    state->shared_mem_size = state->spmm.shared_mem_size; // the figures of the middle (SpMM) launch
+    state->grid_dim[0] = state->spmm.grid_dim[0];
+    state->block_dim[0] = state->spmm.block_dim[0];
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
+int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                               const void* IFMap, void* OFMap, int variant)
+{
+    int frc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
+    if (frc != SHFLBW_OK) return frc;
+    const int Ho = state->Ho, Wo = state->Wo;
+    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
     const long npix = (long)B * Ho * Wo;
     // The scratch cache is bookkeeping of the handle, not part of the weight's value; it is the one member an
     // init call changes, under its lock.
@@ -385,32 +461,19 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         *fresh = true;
         return ptr;
     };
-    auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
     if (variant == 0) {
         // plane form: geometry of the phase planes (see spconv_gfx950.hip)
-        const int s = stride, ph = f->R / 2, pw = f->S / 2;
-        const long PH = (H + 2 * ph + s - 1) / s;
-        const long PW = ((W + 2 * pw + s - 1) / s + 7) / 8 * 8;
-        const long np = (long)B * PH * PW;                                   // plane positions = GEMM columns
-        const long max_shift = (long)((f->R - 1) / s) * PW + (f->S - 1) / s; // largest tap offset
-        const long pitch = (np + max_shift + 8 + 63) / 64 * 64;
-        const int copies = (f->S - 1) / s >= 1 ? 2 : 1;
-        if (copies * s * s > 32) {
-            set_error("spconv_init: stride %d has too many phase planes for the plane form", s);
-            return SHFLBW_ERR_UNSUPPORTED;
-        }
-        const long rows = (long)copies * s * s * f->C; // channel rows of the plane tensor
-        if (np > 0x7fffffffL || (unsigned long long)rows * (unsigned long long)pitch * 2ull > 0xffffffffull) {
-            set_error("spconv_init: problem too large for the plane form (%ld rows of %ld positions)", rows, pitch);
-            return SHFLBW_ERR_UNSUPPORTED;
-        }
-        const size_t slots = f->packed_indices.size();
-        const size_t planes_bytes = up256((size_t)rows * pitch * 2), dm_bytes = up256((size_t)f->F * np * 2);
-        const size_t ids_bytes = up256(slots * sizeof(int) + 64);
+        PlaneForm g;
+        int grc = plane_form_geometry(f, B, H, W, stride, &g);
+        if (grc != SHFLBW_OK) return grc;
+        const int s = stride;
+        const long PW = g.PW, pitch = g.pitch;
+        const int copies = g.copies;
+        const size_t slots = g.slots, planes_bytes = g.planes_bytes, dm_bytes = g.dm_bytes, ids_bytes = g.ids_bytes;
         bool fresh = false;
-        char* scratch = (char*)cached_scratch(planes_bytes + dm_bytes + 2 * ids_bytes, &fresh);
+        char* scratch = (char*)cached_scratch(g.total_bytes(), &fresh);
         if (!scratch) {
-            set_error("spconv_init: cannot allocate %zu bytes of device scratch", planes_bytes + dm_bytes + 2 * ids_bytes);
+            set_error("spconv_init: cannot allocate %zu bytes of device scratch", g.total_bytes());
             return SHFLBW_ERR_HIP;
         }
         int* d_ids = (int*)(scratch + planes_bytes + dm_bytes);
@@ -437,20 +500,7 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
             SHFLBW_HIP_TRY(hipMemcpy(d_ids, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
             SHFLBW_HIP_TRY(hipMemcpy(d_ids_pm, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
         }
-        state->planes = scratch;
-        state->result_fm = scratch + planes_bytes;
-        state->np = (int)np;
-        state->plane_rows = (int)PH;
-        state->plane_cols = (int)PW;
-        state->plane_pitch = (int)pitch;
-        state->plane_copies = copies;
-        int rc = shflbw_spmm_init(&state->spmm, f, (int)np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
-        if (rc != SHFLBW_OK) return rc;
-        // the gather walks the planes: ids are element offsets, one id apart is one value apart
-        state->spmm.packed_indices = d_ids;
-        state->spmm.packed_indices_pm = d_ids_pm;
-        state->spmm.ldb_bytes = 2;
-        state->spmm.args.K = (int)(rows * pitch); // extent of the id space
+        return bind_plane_form(state, f, g, scratch);
     }
     if (variant == 2) {
         // im2col form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
@@ -556,6 +606,73 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         return SHFLBW_ERR_HIP;
     }
     return SHFLBW_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The entry point that allocates nothing: the scratch of the plane form in a fixed device array.
+// `scratch` below is only the host-side handle of the symbol; the device address of each GPU's copy
+// comes from hipGetSymbolAddress, once per device, and only that address is handed to kernels.
+// ---------------------------------------------------------------------------------------------------
+} // extern "C"
+
+static __device__ __align__(256) unsigned char scratch[SHFLBW_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_static_lock;
+void* g_static_addr[kMaxDevices] = {};
+
+// device address of this GPU's copy of `scratch` (looked up on the first call with that device current)
+int static_scratch_address(char** out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("spconv_exec_static: cannot tell the current device");
+        return SHFLBW_ERR_HIP;
+    }
+    std::lock_guard<std::mutex> guard(g_static_lock);
+    if (!g_static_addr[dev]) {
+        void* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_error("spconv_exec_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        g_static_addr[dev] = ptr;
+    }
+    *out = (char*)g_static_addr[dev];
+    return SHFLBW_OK;
+}
+} // namespace
+
+extern "C" {
+
+int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int stride, const void* IFMap, void* OFMap,
+                              void* stream)
+{
+    shflbw_spconv_state st;
+    int rc = spconv_fill_state(&st, f, B, H, W, stride, IFMap, OFMap, 0);
+    if (rc != SHFLBW_OK) return rc;
+    PlaneForm g;
+    if ((rc = plane_form_geometry(f, B, H, W, stride, &g)) != SHFLBW_OK) return rc;
+    if (g.total_bytes() > (size_t)SHFLBW_STATIC_SCRATCH_BYTES) {
+        set_error("spconv_exec_static: this problem needs %zu bytes of scratch, the fixed array holds %zu", g.total_bytes(),
+                  (size_t)SHFLBW_STATIC_SCRATCH_BYTES);
+        return SHFLBW_ERR_CAPACITY;
+    }
+    char* base = nullptr;
+    if ((rc = static_scratch_address(&base)) != SHFLBW_OK) return rc;
+    // Nothing in the array has to start at zero: the layout pass writes every plane position a pixel's taps
+    // read (zeros outside the image), the rest only feeds plane positions that are no output pixel.
+    if ((rc = bind_plane_form(&st, f, g, base)) != SHFLBW_OK) return rc;
+    hipError_t e = launch_plane_ids((const int*)f->d_packed_indices, (int*)(base + g.planes_bytes + g.dm_bytes),
+                                    (int*)(base + g.planes_bytes + g.dm_bytes + g.ids_bytes), (int)g.slots, f->C, f->S,
+                                    stride, g.PW, (int)g.pitch, g.copies, (hipStream_t)stream);
+    if (e != hipSuccess) {
+        set_error("spconv_exec_static: id launch failed: %s", hipGetErrorString(e));
+        return SHFLBW_ERR_HIP;
+    }
+    return shflbw_spconv_exec(&st, stream);
 }
 
 static const char* const g_spconv_forms[] = {

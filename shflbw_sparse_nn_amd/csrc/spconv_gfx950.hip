@@ -344,6 +344,35 @@ __global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __res
         });
 }
 
+// Kept-column ids of the packed image (k = (r*S + t)*C + c per slot) -> element offsets into the plane
+// tensor, in slot order and in the producer-major order of every 64-slot group; the device-side twin of
+// the rewrite shflbw_spconv_init does on the host.
+__global__ void __launch_bounds__(256) plane_ids_kernel(const int* __restrict__ kidx, int* __restrict__ ids,
+                                                        int* __restrict__ ids_pm, int slots, int C, int S, int stride,
+                                                        int PW, int pitch, int copies)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= slots) return;
+    const int k = kidx[q];
+    const int c = k % C, tap = k / C, r = tap / S, t = tap % S;
+    const int shift = (r / stride) * PW + t / stride;
+    const int copy = copies == 2 ? (shift & 1) : 0;
+    const int phase = (r % stride) * stride + t % stride;
+    const int id = ((copy * stride * stride + phase) * C + c) * pitch + shift - copy;
+    ids[q] = id;
+    const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, rr = q % 4;
+    ids_pm[grp * 64 + 16 * p + 4 * j + rr] = id;
+}
+
+hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, int C, int S, int stride, int PW,
+                            int pitch, int copies, hipStream_t stream)
+{
+    if (slots <= 0) return hipSuccess;
+    hipLaunchKernelGGL(plane_ids_kernel, dim3((slots + 255) / 256), dim3(256), 0, stream, kidx, ids, ids_pm, slots, C, S,
+                       stride, PW, pitch, copies);
+    return hipGetLastError();
+}
+
 hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int PH, int PW, int pitch, int copies,
                                  hipStream_t stream)
 {

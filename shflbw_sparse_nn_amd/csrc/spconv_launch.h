@@ -37,6 +37,11 @@ hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int 
 hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, int B, int PH, int PW, int Ho, int Wo,
                                  hipStream_t stream);
 
+// Plane-form ids computed on the device (for callers that may not copy from the host): slot-ordered and
+// producer-major element offsets from the packed kept-column ids.
+hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, int C, int S, int stride, int PW,
+                            int pitch, int copies, hipStream_t stream);
+
 // Stages 1 and 3 of the im2col form of the convolution: NHWC input -> im2col matrix with rows of NP
 // halves (NP a multiple of 64), and filter-major result -> NHWC output.
 hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream);
