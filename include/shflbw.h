@@ -229,6 +229,8 @@ typedef struct shflbw_spconv_state {
     int np;
     void* planes;
     int plane_rows, plane_cols, plane_pitch, plane_copies;
+    int ncols;  /* fused form: columns of the GEMM = plane positions of output rows, B*Ho*plane_cols; result_fm is [F][ncols] */
+    void* sync; /* fused form: synchronisation words in the scratch, all zero between launches */
     shflbw_spmm_state spmm;
 } shflbw_spconv_state;
 

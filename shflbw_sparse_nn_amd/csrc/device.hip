@@ -4,7 +4,9 @@
 // block_sparse/spconv/blockwise_op.h:79-193 (init / exec).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -139,8 +141,10 @@ struct PlaneForm {
     long pitch;     // values per channel row of the plane tensor
     long rows;      // channel rows: copies * stride^2 * C
     size_t slots;   // padded kept-vector slots of the filter
-    size_t planes_bytes, dm_bytes, ids_bytes; // scratch = planes | result_fm | ids | ids_pm
-    size_t total_bytes() const { return planes_bytes + dm_bytes + 2 * ids_bytes; }
+    long ncols;     // columns of the fused form: plane positions of output rows only, B * Ho * PW
+    int Ho, Wo;
+    size_t planes_bytes, dm_bytes, ids_bytes, sync_bytes; // scratch = planes | result_fm | ids | ids_pm | sync words
+    size_t total_bytes() const { return planes_bytes + dm_bytes + 2 * ids_bytes + sync_bytes; }
 };
 
 static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int stride, PlaneForm* g)
@@ -166,7 +170,40 @@ static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int 
     g->planes_bytes = up256((size_t)g->rows * g->pitch * 2);
     g->dm_bytes = up256((size_t)f->F * g->np * 2);
     g->ids_bytes = up256(g->slots * sizeof(int) + 64);
+    g->Ho = (H + 2 * ph - f->R) / s + 1;
+    g->Wo = (W + 2 * pw - f->S) / s + 1;
+    g->ncols = (long)B * g->Ho * g->PW;
+    g->sync_bytes = (size_t)conv_sync_lines((int)((g->ncols + 255) / 256)) * SYNC_LINE * sizeof(int); // column tiles are 256 wide at least
     return SHFLBW_OK;
+}
+
+// launch arguments of the SpMM kernels from a state; BN is the tile width of the kernel that will run
+static void fill_spmm_launch_args(const shflbw_spmm_state* state, int BN, SpmmLaunchArgs* out)
+{
+    SpmmLaunchArgs& a = *out;
+    a.M = state->args.M;
+    a.N = state->args.N;
+    a.K = state->args.K;
+    a.X = a.M / state->brow;
+    a.n_tiles = 0;
+    a.packedA = (const half8_t*)state->packed_values;
+    a.kidx = state->packed_indices;
+    a.kidx_pm = state->packed_indices_pm;
+    a.panel_desc = state->panel_ptr;
+    a.row_ids = state->args.A_row_indices;
+    a.B = (const half_t*)state->args.B;
+    a.ldb_bytes = state->ldb_bytes;
+    a.C = (const half_t*)state->args.C;
+    a.D = (half_t*)state->args.D;
+    a.alpha = state->args.alpha;
+    a.beta = state->args.beta;
+    a.num_cus = device_compute_units();
+    a.img_cols = 1, a.img_skip = 0;
+    a.tile_arrivals = nullptr;
+    // rows of B one column tile can touch: above about 2.5 MB they do not stay in the 4 MB L2 of an XCD
+    // from one round of tiles to the next, and alternating the direction of the walk pays (measured:
+    // +1 % at 2 MB, -4 % at 3 MB, -7 % at 4 MB, -13 % at 8 MB)
+    a.alternate = (double)a.K * a.ldb_bytes * BN / (a.N > 0 ? a.N : 1) > 2.5 * 1024 * 1024;
 }
 
 } // namespace shflbw
@@ -288,27 +325,7 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
     const SpmmVariant* v = find_spmm_variant(state->brow, state->variant, nullptr);
     if (!v) return SHFLBW_ERR_UNSUPPORTED;
     SpmmLaunchArgs a;
-    a.M = state->args.M;
-    a.N = state->args.N;
-    a.K = state->args.K;
-    a.X = a.M / state->brow;
-    a.n_tiles = 0;
-    a.packedA = (const half8_t*)state->packed_values;
-    a.kidx = state->packed_indices;
-    a.kidx_pm = state->packed_indices_pm;
-    a.panel_desc = state->panel_ptr;
-    a.row_ids = state->args.A_row_indices;
-    a.B = (const half_t*)state->args.B;
-    a.ldb_bytes = state->ldb_bytes;
-    a.C = (const half_t*)state->args.C;
-    a.D = (half_t*)state->args.D;
-    a.alpha = state->args.alpha;
-    a.beta = state->args.beta;
-    a.num_cus = device_compute_units();
-    // rows of B one column tile can touch: above about 2.5 MB they do not stay in the 4 MB L2 of an XCD
-    // from one round of tiles to the next, and alternating the direction of the walk pays (measured:
-    // +1 % at 2 MB, -4 % at 3 MB, -7 % at 4 MB, -13 % at 8 MB)
-    a.alternate = (double)a.K * a.ldb_bytes * v->BN / (a.N > 0 ? a.N : 1) > 2.5 * 1024 * 1024;
+    fill_spmm_launch_args(state, v->BN, &a);
     if (a.X == 0) return SHFLBW_OK;
     hipError_t e = v->launch(a, (hipStream_t)stream);
     if (e != hipSuccess) {
@@ -317,6 +334,7 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
     }
     return SHFLBW_OK;
 }
+
 
 int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
                        const void* IFMap, void* OFMap)
@@ -365,7 +383,7 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
         return SHFLBW_ERR_SHAPE;
     }
     if (variant < 0 || variant >= shflbw_spconv_variant_count()) {
-        set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = im2col form)", variant);
+        set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = im2col form, 3 = plane form fused into one launch)", variant);
         return SHFLBW_ERR_INVALID;
     }
     const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
@@ -410,7 +428,8 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
 
 // Points a state of the plane form at its scratch (planes | result_fm | ids | ids_pm, laid out by `g`) and sets
 // up the SpMM launch in the middle.  The ids must be in the scratch when the state is executed.
-static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, const PlaneForm& g, char* scratch)
+static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, const PlaneForm& g, char* scratch,
+                           bool fused)
 {
     state->planes = scratch;
     state->result_fm = scratch + g.planes_bytes;
@@ -419,8 +438,23 @@ static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, c
     state->plane_cols = g.PW;
     state->plane_pitch = (int)g.pitch;
     state->plane_copies = g.copies;
-    int rc = shflbw_spmm_init(&state->spmm, f, (int)g.np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
+    state->ncols = (int)g.ncols;
+    state->sync = scratch + g.planes_bytes + g.dm_bytes + 2 * g.ids_bytes;
+    // the three-launch form computes every plane position, the fused form only those of output rows
+    int rc = fused ? shflbw_spmm_init_variant(&state->spmm, f, (int)g.ncols, state->planes, nullptr, state->result_fm, 1.f, 0.f, 0)
+                   : shflbw_spmm_init(&state->spmm, f, (int)g.np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
     if (rc != SHFLBW_OK) return rc;
+    if (fused) {
+        const ConvFusedKernel* k = conv_fused_kernel(f->brow);
+        if (!k) {
+            set_error("spconv_init: no fused kernel for block size %d", f->brow);
+            return SHFLBW_ERR_UNSUPPORTED;
+        }
+        SHFLBW_HIP_TRY(k->prepare());
+        state->spmm.shared_mem_size = (size_t)k->lds_bytes;
+        state->spmm.grid_dim[0] = (unsigned)((f->nrow / f->brow) * ((g.ncols + k->BN - 1) / k->BN));
+        state->spmm.block_dim[0] = (unsigned)k->threads;
+    }
     // the gather walks the planes: ids are element offsets, one id apart is one value apart
     state->spmm.packed_indices = (const int*)(scratch + g.planes_bytes + g.dm_bytes);
     state->spmm.packed_indices_pm = (const int*)(scratch + g.planes_bytes + g.dm_bytes + g.ids_bytes);
@@ -461,8 +495,8 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         *fresh = true;
         return ptr;
     };
-    if (variant == 0) {
-        // plane form: geometry of the phase planes (see spconv_gfx950.hip)
+    if (variant == 0 || variant == 3) {
+        // plane forms: geometry of the phase planes (see spconv_gfx950.hip)
         PlaneForm g;
         int grc = plane_form_geometry(f, B, H, W, stride, &g);
         if (grc != SHFLBW_OK) return grc;
@@ -482,6 +516,8 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
             // the tail of every channel row and the positions no image covers are read (for results
             // nobody uses) but never written
             SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes));
+            // the synchronisation words of the fused form start at zero (every launch leaves them so)
+            SHFLBW_HIP_TRY(hipMemset(scratch + planes_bytes + dm_bytes + 2 * ids_bytes, 0, g.sync_bytes));
             // kept-column id k = (r*S + t)*C + c  ->  element offset of (copy, phase, channel) row + tap offset
             std::vector<int> ids(slots), ids_pm(slots);
             for (size_t q = 0; q < slots; q++) {
@@ -500,7 +536,7 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
             SHFLBW_HIP_TRY(hipMemcpy(d_ids, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
             SHFLBW_HIP_TRY(hipMemcpy(d_ids_pm, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
         }
-        return bind_plane_form(state, f, g, scratch);
+        return bind_plane_form(state, f, g, scratch, variant == 3);
     }
     if (variant == 2) {
         // im2col form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
@@ -567,6 +603,75 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
+    if (state->variant == 3) {
+        const ConvFusedKernel* k = conv_fused_kernel(state->brow);
+        if (!k) return SHFLBW_ERR_UNSUPPORTED;
+        SpmmLaunchArgs m;
+        fill_spmm_launch_args(&state->spmm, k->BN, &m);
+        if (m.X == 0) return SHFLBW_OK;
+        m.alternate = 0; // the planes under one column tile are far smaller than an L2
+        m.img_cols = a.Ho * state->plane_cols;
+        m.img_skip = (state->plane_rows - a.Ho) * state->plane_cols;
+        m.tile_arrivals = (int*)state->sync + CONV_LINE_SLAB0 * SYNC_LINE;
+        ConvFuseArgs c;
+        c.g = PlaneGeom{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, state->plane_rows, state->plane_cols,
+                        state->plane_pitch, state->plane_copies, 0, {}};
+        if (!fill_wanted_planes(c.g, a.R, a.S)) return SHFLBW_ERR_UNSUPPORTED;
+        // chunks of the two layout phases: 8, 4 or 2 tiles of 64 x 64, the largest size that still gives every
+        // workgroup a chunk; along the contiguous axis of the source (channels, filters) as many tiles as there are
+        auto pow2_le = [](int n, int cap) { int p = 1; while (p * 2 <= n && p * 2 <= cap) p *= 2; return p; };
+        const int grid = std::min((m.num_cus / 8) * 8, ((m.X * ((state->ncols + k->BN - 1) / k->BN) + 7) / 8) * 8);
+        c.in = a.in;
+        c.planes = (half_t*)state->planes;
+        c.np64 = (state->np + 63) / 64 * 64;
+        for (int tiles = 8; tiles >= 2; tiles >>= 1) {
+            c.ct = pow2_le((a.C + 63) / 64, tiles);
+            c.pt = tiles / c.ct;
+            c.ch_chunks = (a.C + c.ct * 64 - 1) / (c.ct * 64);
+            c.pos_chunks = (c.np64 + c.pt * 64 - 1) / (c.pt * 64);
+            c.n0chunks = c.g.nwanted * c.ch_chunks * c.pos_chunks;
+            if (c.n0chunks >= grid) break;
+        }
+        c.fm = (const half_t*)state->result_fm;
+        c.out = a.out;
+        c.F = a.F;
+        c.ncols = state->ncols;
+        c.Ho = a.Ho;
+        c.Wo = a.Wo;
+        for (int tiles = 8; tiles >= 2; tiles >>= 1) {
+            c.ft = pow2_le((a.F + 63) / 64, tiles);
+            c.mt = tiles / c.ft;
+            c.f_chunks = (a.F + c.ft * 64 - 1) / (c.ft * 64);
+            if (c.f_chunks * ((k->BN / 64 + c.mt - 1) / c.mt) >= m.X) break; // a chunk for every workgroup of a column tile
+        }
+        c.slabs = (state->ncols + k->BN - 1) / k->BN;
+        c.arrivals_per_slab = m.X;
+        c.sync = (int*)state->sync;
+        c.magic_ps = udiv_magic(state->plane_rows * state->plane_cols);
+        c.magic_pw = udiv_magic(state->plane_cols);
+        c.magic_imgcols = udiv_magic(a.Ho * state->plane_cols);
+        c.help_ticks = 3000; // 30 us
+        // Measurement knob: SHFLBW_FUSED_PHASES (bit 0: input rewrite inside the launch, bit 1: NHWC output inside
+        // the launch; default 3).  A cleared bit runs that step as its own launch around the fused kernel.
+        static const int phases = [] {
+            const char* e = getenv("SHFLBW_FUSED_PHASES");
+            return e ? atoi(e) & 3 : 3;
+        }();
+        c.phases = phases;
+        hipError_t e = hipSuccess;
+        if (!(phases & 1))
+            e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols, state->plane_pitch,
+                                      state->plane_copies, (hipStream_t)stream);
+        if (e == hipSuccess) e = k->launch(m, c, (hipStream_t)stream);
+        if (e == hipSuccess && !(phases & 2)) // the compact result has Ho rows per image
+            e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, state->ncols, a.B, a.Ho,
+                                      state->plane_cols, a.Ho, a.Wo, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: fused launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        return SHFLBW_OK;
+    }
     if (state->variant == 0) {
         hipError_t e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
                                              state->plane_pitch, state->plane_copies, (hipStream_t)stream);
@@ -664,7 +769,7 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
     if ((rc = static_scratch_address(&base)) != SHFLBW_OK) return rc;
     // Nothing in the array has to start at zero: the layout pass writes every plane position a pixel's taps
     // read (zeros outside the image), the rest only feeds plane positions that are no output pixel.
-    if ((rc = bind_plane_form(&st, f, g, base)) != SHFLBW_OK) return rc;
+    if ((rc = bind_plane_form(&st, f, g, base, false)) != SHFLBW_OK) return rc;
     hipError_t e = launch_plane_ids((const int*)f->d_packed_indices, (int*)(base + g.planes_bytes + g.dm_bytes),
                                     (int*)(base + g.planes_bytes + g.dm_bytes + g.ids_bytes), (int)g.slots, f->C, f->S,
                                     stride, g.PW, (int)g.pitch, g.copies, (hipStream_t)stream);
@@ -676,9 +781,10 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
 }
 
 static const char* const g_spconv_forms[] = {
-    "planes+spmm+transpose",  // 0: NHWC -> channel-major planes, SpMM gather with tap offsets, transpose to NHWC
+    "planes+spmm+transpose",  // 0: NHWC -> channel-major planes, SpMM gather with tap offsets, transpose to NHWC: three launches
     "direct",                 // 1: one kernel, im2col gather from NHWC in the tile loads
-    "im2col+spmm+transpose",  // 2: explicit im2col matrix
+    "im2col+spmm+transpose",  // 2: explicit im2col matrix, three launches
+    "fused-planes",           // 3: the steps of form 0 in one persistent launch
 };
 
 int shflbw_spconv_variant_count(void) { return (int)(sizeof(g_spconv_forms) / sizeof(g_spconv_forms[0])); }

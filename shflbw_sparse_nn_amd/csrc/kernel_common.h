@@ -94,6 +94,10 @@ __device__ __forceinline__ void store_result_16B(half_t* p, half8_t v)
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
+// Words that workgroups of one launch count in (queues, arrival counts) are kept one cache line apart: atomics on
+// one line are served one after the other (about 11 ns each with every compute unit taking part).
+constexpr int SYNC_LINE = 64; // ints
+
 // Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs; this makes consecutive *logical* ids share an XCD (and
 // therefore its L2), so tiles that gather the same activation slab run side by side.

@@ -11,6 +11,7 @@
 // matrix-core part (transposing LDS loads, 32x32x16 fp16 MFMA, fp32 accumulate) is shared.
 #include "kernel_common.h"
 #include "spconv_launch.h"
+#include "spmm_ws.h"
 
 namespace shflbw {
 
@@ -286,14 +287,6 @@ __global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __
 //      are no output pixel (i >= Ho or j >= Wo) compute values nobody reads.
 //   3. planes_to_nhwc_kernel: Dm[f][n'] -> OFMap[pixel][f] for the positions that are pixels.
 // =======================================================================================
-struct PlaneGeom {
-    int B, H, W, C, stride, pad_h, pad_w;
-    int PH, PW;   // rows and (padded) columns of a phase plane
-    int pitch;    // values per channel row of the plane tensor
-    int copies;   // 1, or 2 with the copy moved by one value
-    int nwanted;  // (copy, phase) planes some tap reads; the others are never written
-    unsigned char wanted[32]; // copy * stride * stride + phase of each
-};
 
 // grid: (position tiles, channel tiles, wanted planes); block 256
 __global__ void __launch_bounds__(256) nhwc_to_planes_kernel(const half_t* __restrict__ in, half_t* __restrict__ planes,
@@ -344,6 +337,321 @@ __global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __res
         });
 }
 
+// the (copy, phase) planes some tap reads: tap (r, t) -> phase (r % s, t % s), copy = parity of its offset when
+// there are two copies
+bool fill_wanted_planes(PlaneGeom& g, int R, int S)
+{
+    const int s = g.stride, nphase = s * s;
+    if (g.copies * nphase > (int)sizeof(g.wanted)) return false;
+    bool want[32] = {};
+    for (int r = 0; r < R; r++)
+        for (int t = 0; t < S; t++) {
+            const int shift = (r / s) * g.PW + t / s;
+            want[(g.copies == 2 ? (shift & 1) : 0) * nphase + (r % s) * s + t % s] = true;
+        }
+    g.nwanted = 0;
+    for (int i = 0; i < g.copies * nphase; i++)
+        if (want[i]) g.wanted[g.nwanted++] = (unsigned char)i;
+    return true;
+}
+
+// =======================================================================================
+// Fused form of the convolution: ONE persistent launch.
+//   phase 0  every workgroup takes chunks of the NHWC -> planes rewrite from a queue (64 x 64 tile transposes,
+//            eight tiles at a time) until the queue is empty, then waits until all chunks have been written;
+//   phase 1  the role-split SpMM over its tiles (gather ids are plane offsets; the columns of the GEMM are the
+//            plane positions of output rows only: m = (img * Ho + i) * PW + j), result rows of fp16 in the
+//            filter-major scratch fm[f][m]; every consumer wave counts its finished tile in the arrival word of
+//            the tile's column tile;
+//   phase 2  when all tiles of a column tile have arrived, its fm[F][BN] slab is transposed to NHWC in chunks
+//            taken from that column tile's queue.
+// No wait depends on a workgroup that is not running: phase 0 waits only for chunks that running workgroups
+// have claimed; in phase 2 the workgroup whose arrival completes a column tile finds it complete when it gets
+// there and empties its queue (alone, if it must), every other wait is bounded by a time budget and only adds
+// helpers.  The words in `sync` are all zero between launches: the last workgroup to leave clears them.
+// Data written by one workgroup and read by another (planes, fm) is stored with device scope, followed by a
+// wait for the acknowledgement and an arrival count; the reader passes an acquire fence after it has seen
+// the count.
+// =======================================================================================
+
+// Layout of the synchronisation words, in cache lines of SYNC_LINE ints (conv_sync_lines() of them): line 0 the XCDs
+// whose workgroups have all left, line 1 a flag (a wait that cannot time out did), lines 2.. the eight phase-0 queues,
+// then per queue the chunks of it that are written, then per XCD the workgroups that have left, then the number of
+// phase-0 queues whose chunks are all written, then two lines per column tile: finished tiles, phase-2 queue.
+constexpr int LINE_LEFT_ALL = 0, LINE_GAVE_UP = 1, LINE_Q0 = 2, LINE_DONE0 = 10, LINE_LEFT = 18, LINE_ALLDONE0 = 26,
+              LINE_SLAB0 = CONV_LINE_SLAB0;
+
+// Diagnostic build (-DSHFLBW_CONV_STAMPS): workgroups 0 and 100 leave 100 MHz timestamps of their phase boundaries
+// in the flag line of the synchronisation words (ints 16.. of line 1).
+#ifdef SHFLBW_CONV_STAMPS
+#define CONV_STAMP(i)                                                                                           \
+    do {                                                                                                        \
+        if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100))                                                 \
+            ((unsigned long long*)(c.sync + LINE_GAVE_UP * SYNC_LINE + 16))[(blockIdx.x == 0 ? 0 : 12) + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define CONV_STAMP(i) do { } while (0)
+#endif
+
+// n / d and n % d for n < 2^31 with magic = floor(2^32 / d) computed on the host (udiv_magic): the product's high word
+// is the quotient or one less, one correction step settles it; an integer division by a run-time value costs about
+// forty instructions, and the layout phases do several per 16-byte piece
+__device__ __forceinline__ void fast_divmod(int n, int d, unsigned magic, int& q, int& r)
+{
+    q = (int)__umulhi((unsigned)n, magic);
+    r = n - q * d;
+    if (r >= d) {
+        q++;
+        r -= d;
+    }
+}
+
+__device__ __forceinline__ int sync_load(const int* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// 512 threads transpose 2 * nk (nk = 1, 2 or 4) 64 x 64 fp16 tiles through LDS at `lds` (8 KiB per tile):
+// `load(tile, i, j)` returns the 16-byte piece j (8 halves) of source row i of a tile; `store(tile, o, q, v)` receives
+// the halves at source rows 8q .. 8q+7 of source column o.  Threads 0..255 own tiles 0..nk-1, threads 256..511 tiles
+// nk..2nk-1; all loads of a thread are in flight before the first one is used.  Piece j of row i sits at piece
+// position j ^ (i / 8) of its LDS row, so the eight row groups a wave reads in one instruction fall into eight
+// different bank groups.
+template <typename Load, typename Store>
+__device__ __forceinline__ void transpose_tiles(uint32_t lds, int tid, int nk, Load load, Store store)
+{
+    const int half = tid >> 8, t = tid & 255;
+    half8_t v[4][2];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (k < nk) {
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) v[k][pass] = load(half * nk + k, (t >> 3) + pass * 32, t & 7);
+        }
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (k < nk) {
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const int i = (t >> 3) + pass * 32, j = t & 7;
+                *(SHFLBW_LDS half8_t*)(uintptr_t)(lds + (half * nk + k) * (TT * TT * 2) + i * (TT * 2) + ((j ^ ((i >> 3) & 7)) << 4)) =
+                    v[k][pass];
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (k < nk) {
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const int o = (t >> 3) + pass * 32, q = t & 7;
+                const int c = (((o >> 3) ^ q) << 3) | (o & 7);
+                half8_t r;
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    r[e] = *(SHFLBW_LDS half_t*)(uintptr_t)(lds + (half * nk + k) * (TT * TT * 2) + (q * 8 + e) * (TT * 2) + c * 2);
+                store(half * nk + k, o, q, r);
+            }
+        }
+    __syncthreads();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+__global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_fused_kernel(SpmmLaunchArgs a, ConvFuseArgs c)
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    static_assert((NCONS + NPROD) * 64 == 512 && Cfg::RING_BYTES >= 8 * TT * TT * 2, "the layout phases use 512 threads and up to 64 KiB");
+    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+    __shared__ int mailbox[2];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int X = a.X;
+    if (tid == 0) *(SHFLBW_LDS unsigned*)(uintptr_t)(lds0 + Cfg::LDS_BYTES) = 0u; // consumer waves count finished tiles here
+    __syncthreads();
+    CONV_STAMP(0);
+
+    // ================= phase 0: NHWC input -> channel-major padded planes =================
+    if (c.phases & 1) {
+        const PlaneGeom& g = c.g;
+        const int nphase = g.stride * g.stride, PS = g.PH * g.PW;
+        // The chunk list is cut into eight ranges with a queue each; a workgroup serves the queue of its XCD first and
+        // then the others (a queue that a load shows to be exhausted is skipped without an atomic).  A chunk is written
+        // once its stores are acknowledged; the workgroup that writes the last chunk of a queue counts the queue.
+        const int per_q = (c.n0chunks + 7) >> 3;
+        const int xcd = blockIdx.x & 7;
+        const int nk = (c.ct * c.pt) >> 1;
+        int tried = 0;
+        while (true) {
+            if (tid == 0) {
+                int chunk = -1;
+                while (tried < 8) {
+                    const int qi = (xcd + tried) & 7;
+                    const int lo = qi * per_q, size = min(c.n0chunks, lo + per_q) - lo;
+                    int* q = c.sync + (LINE_Q0 + qi) * SYNC_LINE;
+                    if (size > 0 && sync_load(q) < size) {
+                        const int got = __hip_atomic_fetch_add(q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (got < size) {
+                            chunk = lo + got;
+                            break;
+                        }
+                    }
+                    tried++;
+                }
+                mailbox[0] = chunk;
+            }
+            __syncthreads();
+            const int chunk = __builtin_amdgcn_readfirstlane(mailbox[0]);
+            if (chunk < 0) break;
+            const int plane = chunk / (c.ch_chunks * c.pos_chunks), rem = chunk % (c.ch_chunks * c.pos_chunks);
+            const int p_base = (rem / c.ch_chunks) * (c.pt * TT), c_base = (rem % c.ch_chunks) * (c.ct * TT);
+            const int copy = g.wanted[plane] / nphase, phase = g.wanted[plane] % nphase;
+            const int pa = phase / g.stride, pb = phase % g.stride;
+            half_t* dst = c.planes + ((size_t)(copy * nphase + phase) * g.C) * g.pitch;
+            transpose_tiles(
+                lds0, tid, nk,
+                [&](int tile, int i, int j) { // source row = position (+ copy), piece = 8 channels
+                    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const int n = p_base + (tile / c.ct) * TT + i + copy;
+                    const int ch = c_base + (tile % c.ct) * TT + j * 8;
+                    int img, r2, prow, pcol;
+                    fast_divmod(n, PS, c.magic_ps, img, r2);
+                    fast_divmod(r2, g.PW, c.magic_pw, prow, pcol);
+                    const int hi = prow * g.stride + pa - g.pad_h, wi = pcol * g.stride + pb - g.pad_w;
+                    if (img < g.B && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && ch < g.C)
+                        v = *(const half8_t*)(c.in + ((size_t)(img * g.H + hi) * g.W + wi) * g.C + ch);
+                    return v;
+                },
+                [&](int tile, int o, int q, half8_t v) { // destination row = channel, 8 positions
+                    const int ch = c_base + (tile % c.ct) * TT + o;
+                    const int p = p_base + (tile / c.ct) * TT + q * 8;
+                    if (ch < g.C && p < c.np64) store_result_16B(dst + (size_t)ch * g.pitch + p, v);
+                });
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                const int qi = min(chunk / per_q, 7), size = min(c.n0chunks, (qi + 1) * per_q) - qi * per_q;
+                if (__hip_atomic_fetch_add(c.sync + (LINE_DONE0 + qi) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == size - 1)
+                    __hip_atomic_fetch_add(c.sync + LINE_ALLDONE0 * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        CONV_STAMP(1);
+        CONV_STAMP(2);
+        // Wait until every queue is written.  The planes were not read by this launch so far, so no cache holds lines of
+        // them except the up-to-date ones of their writers (caches start a launch invalidated, and the stores go through
+        // to memory): the gathers that follow need no invalidation of their own.
+        if (tid == 0) {
+            const int queues = (c.n0chunks + per_q - 1) / max(per_q, 1);
+            const unsigned long long t0 = wall_clock64();
+            while (sync_load(c.sync + LINE_ALLDONE0 * SYNC_LINE) < queues) {
+                if (wall_clock64() - t0 > 200000000ull) { // two seconds: cannot happen, chunks are only held by running workgroups
+                    __hip_atomic_store(c.sync + LINE_GAVE_UP * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
+        }
+        __syncthreads();
+        CONV_STAMP(3);
+        CONV_STAMP(4);
+    }
+
+    // ================= phase 1: the SpMM over this workgroup's tiles =================
+    const int T = X * a.n_tiles;
+    const int per = (T + 7) >> 3;
+    const int S = gridDim.x >> 3;
+    const int id_first = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    const int id_end = min(T, ((blockIdx.x & 7) + 1) * per);
+    {
+        if (wave >= NCONS)
+            ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE, true>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
+        else if constexpr (V == 16)
+            ws_consumer16<Cfg, WN, NCONS, true>(a, lds0, lane, wave, id_first, id_end, S);
+        else
+            ws_consumer<Cfg, V, WN, NCONS, true>(a, lds0, lane, wave, id_first, id_end, S);
+    }
+    __syncthreads(); // both roles are through: the ring is free
+    CONV_STAMP(5);
+
+    // ================= phase 2: fm[F][BN] slabs -> NHWC output =================
+    if (c.phases & 2) {
+        const int chunks_per_slab = c.f_chunks * ((Cfg::BN / TT + c.mt - 1) / c.mt);
+        const int img_cols = c.Ho * c.g.PW;
+        const unsigned long long t0 = wall_clock64();
+        // One visit to every column tile this workgroup computed a tile of (in its tile order).  A column tile that is
+        // complete is emptied; for one that is not, the workgroup waits while it has time left and moves on otherwise:
+        // the workgroup whose arrival completes it comes by later and empties it.
+        int prev = -1;
+        for (int id = id_first; id < id_end; id += S) {
+            const int s = id / X;
+            if (s == prev) continue;
+            prev = s;
+            if (tid == 0) {
+                int ok = 0;
+                while (true) {
+                    if (sync_load(c.sync + (LINE_SLAB0 + 2 * s) * SYNC_LINE) >= c.arrivals_per_slab) {
+                        ok = 1;
+                        break;
+                    }
+                    if (wall_clock64() - t0 > (unsigned long long)c.help_ticks) break;
+                    __builtin_amdgcn_s_sleep(2);
+                }
+                mailbox[1] = ok;
+            }
+            __syncthreads();
+            const int ok = __builtin_amdgcn_readfirstlane(mailbox[1]);
+            __syncthreads();
+            if (!ok) continue;
+            // the result rows were not read by this launch so far (see the planes above): no invalidation needed
+            CONV_STAMP(6);
+            CONV_STAMP(7);
+            while (true) {
+                if (tid == 0)
+                    mailbox[0] = __hip_atomic_fetch_add(c.sync + (LINE_SLAB0 + 2 * s + 1) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                const int chunk = __builtin_amdgcn_readfirstlane(mailbox[0]);
+                if (chunk >= chunks_per_slab) break;
+                const int f_base = (chunk % c.f_chunks) * (c.ft * TT);
+                const int m_base = s * Cfg::BN + (chunk / c.f_chunks) * (c.mt * TT);
+                const int m_end = min(c.ncols, (s + 1) * Cfg::BN);
+                transpose_tiles(
+                    lds0, tid, (c.ft * c.mt) >> 1,
+                    [&](int tile, int i, int j) { // source row = filter, piece = 8 columns of the GEMM
+                        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                        const int f = f_base + (tile % c.ft) * TT + i;
+                        const int m = m_base + (tile / c.ft) * TT + j * 8;
+                        if (f < c.F && m < m_end) v = *(const half8_t*)(c.fm + (size_t)f * c.ncols + m);
+                        return v;
+                    },
+                    [&](int tile, int o, int q, half8_t v) { // destination row = the pixel of column m, 8 filters
+                        const int m = m_base + (tile / c.ft) * TT + o;
+                        const int f = f_base + (tile % c.ft) * TT + q * 8;
+                        int img, r2, ho, wo;
+                        fast_divmod(m, img_cols, c.magic_imgcols, img, r2);
+                        fast_divmod(r2, c.g.PW, c.magic_pw, ho, wo);
+                        if (m < m_end && wo < c.Wo && f < c.F)
+                            *(half8_t*)(c.out + ((size_t)(img * c.Ho + ho) * c.Wo + wo) * c.F + f) = v;
+                    });
+            }
+        }
+    }
+
+    // ================= leave: the last workgroup clears the words for the next launch =================
+    // counted per XCD first (one line each), then the XCDs on one line
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    CONV_STAMP(8);
+    if (tid == 0) {
+        const int xcd = blockIdx.x & 7, per_xcd = (int)gridDim.x >> 3; // the grid is a multiple of 8
+        if (__hip_atomic_fetch_add(c.sync + (LINE_LEFT + xcd) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == per_xcd - 1 &&
+            __hip_atomic_fetch_add(c.sync + LINE_LEFT_ALL * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 7) {
+            for (int i = 0; i < LINE_SLAB0 + 2 * c.slabs; i++)
+                if (i != LINE_GAVE_UP) __hip_atomic_store(c.sync + i * SYNC_LINE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // Kept-column ids of the packed image (k = (r*S + t)*C + c per slot) -> element offsets into the plane
 // tensor, in slot order and in the producer-major order of every 64-slot group; the device-side twin of
 // the rewrite shflbw_spconv_init does on the host.
@@ -377,17 +685,7 @@ hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int 
                                  hipStream_t stream)
 {
     PlaneGeom g{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, PH, PW, pitch, copies, 0, {}};
-    // the planes the taps read: tap (r, t) -> phase (r % s, t % s), copy = parity of its offset when there are two
-    const int s = a.stride, nphase = s * s;
-    if (copies * nphase > (int)sizeof(g.wanted)) return hipErrorInvalidValue;
-    bool want[32] = {};
-    for (int r = 0; r < a.R; r++)
-        for (int t = 0; t < a.S; t++) {
-            const int shift = (r / s) * PW + t / s;
-            want[(copies == 2 ? (shift & 1) : 0) * nphase + (r % s) * s + t % s] = true;
-        }
-    for (int i = 0; i < copies * nphase; i++)
-        if (want[i]) g.wanted[g.nwanted++] = (unsigned char)i;
+    if (!fill_wanted_planes(g, a.R, a.S)) return hipErrorInvalidValue;
     const int np = a.B * PH * PW;
     const dim3 grid((np + TT - 1) / TT, (a.C + TT - 1) / TT, g.nwanted);
     hipLaunchKernelGGL(nhwc_to_planes_kernel, grid, dim3(256), 0, stream, a.in, planes, g);
@@ -415,6 +713,51 @@ hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int np
     const dim3 grid(NP / TT, (F + TT - 1) / TT);
     hipLaunchKernelGGL(transpose_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, npix, NP);
     return hipGetLastError();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+static hipError_t launch_fused(const SpmmLaunchArgs& a, const ConvFuseArgs& c, hipStream_t stream)
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    SpmmLaunchArgs b = a;
+    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    const int T = a.X * b.n_tiles;
+    int grid = a.num_cus > 0 ? a.num_cus : 256;
+    grid = (grid / 8) * 8;
+    const int need = ((T + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL((spconv_fused_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid), dim3(Cfg::THREADS),
+                       Cfg::LDS_BYTES + 16, stream, b, c);
+    return hipGetLastError();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+static hipError_t prepare_fused()
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    return hipFuncSetAttribute((const void*)spconv_fused_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES + 16);
+}
+
+#define SHFLBW_FUSED(V, WN, NC, NP, KT, NS)                                                                     \
+    {                                                                                                           \
+        V, WN* NC, NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS>::LDS_BYTES + 16, &launch_fused<V, WN, NC, NP, KT, NS>, \
+            &prepare_fused<V, WN, NC, NP, KT, NS>                                                               \
+    }
+
+// one fused kernel per block height: the tile shape of the SpMM default of that height
+static const ConvFusedKernel g_fused[] = {
+    SHFLBW_FUSED(64, 128, 4, 4, 32, 4),
+    SHFLBW_FUSED(32, 128, 4, 4, 32, 4),
+    SHFLBW_FUSED(16, 128, 4, 4, 32, 4),
+    SHFLBW_FUSED(128, 64, 4, 4, 32, 6),
+};
+
+const ConvFusedKernel* conv_fused_kernel(int V)
+{
+    for (const ConvFusedKernel& k : g_fused)
+        if (k.V == V) return &k;
+    return nullptr;
 }
 
 template <int V, int WN, int NWAVES, int KT>

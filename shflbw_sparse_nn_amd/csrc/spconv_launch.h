@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "kernel_common.h"
+#include "spmm_launch.h"
 
 namespace shflbw {
 
@@ -28,6 +29,55 @@ struct SpconvVariant {
 };
 
 const SpconvVariant* spconv_variants(int* count);
+
+// Geometry of the channel-major padded planes the plane forms of the convolution gather from.
+struct PlaneGeom {
+    int B, H, W, C, stride, pad_h, pad_w;
+    int PH, PW;   // rows and (padded) columns of a phase plane
+    int pitch;    // values per channel row of the plane tensor
+    int copies;   // 1, or 2 with the copy moved by one value
+    int nwanted;  // (copy, phase) planes some tap reads; the others are never written
+    unsigned char wanted[32]; // copy * stride * stride + phase of each
+};
+
+bool fill_wanted_planes(PlaneGeom& g, int R, int S);
+
+// Arguments of the fused (single launch) form beside those of the SpMM in its middle.
+struct ConvFuseArgs {
+    PlaneGeom g;          // input side (phase 0)
+    const half_t* in;     // NHWC input
+    half_t* planes;
+    int np64;             // plane positions written per channel row (rounded up to 64)
+    int ct, pt;           // phase-0 chunk: ct channel tiles x pt position tiles of 64 (ct * pt = 8, 4 or 2)
+    int ch_chunks, pos_chunks, n0chunks; // chunks per plane along channels / positions, and in total
+    const half_t* fm;     // [F][ncols] filter-major result (phase 1 output, phase 2 input)
+    half_t* out;          // NHWC output
+    int F, ncols, Ho, Wo;
+    int ft, mt;           // phase-2 chunk: ft filter tiles x mt column tiles of 64 (ft * mt = 8, 4 or 2)
+    int f_chunks;         // chunks per column tile along F
+    int slabs;            // column tiles of the GEMM
+    int arrivals_per_slab; // finished tiles that complete a column tile (one per row panel)
+    int* sync;            // synchronisation words, conv_sync_lines(slabs) cache lines of SYNC_LINE ints, all zero between launches
+    unsigned magic_ps, magic_pw, magic_imgcols; // udiv_magic of PH*PW, PW and Ho*PW
+    int help_ticks;       // 100 MHz ticks a workgroup without obligation keeps waiting for column tiles in phase 2
+    int phases;           // bit 0: run phase 0, bit 1: run phase 2 (cleared: the layout kernels are launched around it)
+};
+
+struct ConvFusedKernel {
+    int V;
+    int BN;      // columns of the GEMM per tile
+    int ncons;   // consumer waves per workgroup (arrivals per tile)
+    int threads;
+    int lds_bytes;
+    hipError_t (*launch)(const SpmmLaunchArgs&, const ConvFuseArgs&, hipStream_t);
+    hipError_t (*prepare)();
+};
+const ConvFusedKernel* conv_fused_kernel(int V);
+// cache lines of synchronisation words the fused form needs for a problem with `slabs` column tiles
+// floor(2^32 / d) for fast_divmod on the device
+inline unsigned udiv_magic(int d) { return d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / (unsigned)d); }
+constexpr int CONV_LINE_SLAB0 = 27; // first of the two lines per column tile
+inline int conv_sync_lines(int slabs) { return CONV_LINE_SLAB0 + 2 * slabs; }
 
 // Stages 1 and 3 of the plane form of the convolution: NHWC input -> channel-major padded planes (one per
 // stride phase, `copies` = 1 or 2 with a copy moved by one value, rows of `pitch` values), and the

@@ -48,7 +48,7 @@ def test_spmm_exec_in_a_graph(torch_gpu):
     _replays(torch, op, [to_dev(torch, B) for B in Bs], dB, dD, refs)
 
 
-@pytest.mark.parametrize("variant", [0, 2])
+@pytest.mark.parametrize("variant", [0, 2, 3])
 def test_spconv_exec_in_a_graph(torch_gpu, variant):
     torch = torch_gpu
     Bn, H, W, C, F, R, Sx, stride, V = 4, 14, 14, 64, 128, 3, 3, 2, 64

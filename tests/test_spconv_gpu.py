@@ -19,8 +19,9 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    # 0: plane layout + SpMM + transpose (default), 1: one direct kernel, 2: im2col matrix + SpMM + transpose
-    for variant in ((0, 1, 2) if V != 16 else (0, 2)):
+    # 0: plane layout + SpMM + transpose (default), 1: one direct kernel, 2: im2col matrix + SpMM + transpose, 3: form 0 fused into one launch
+    for variant in ((0, 3, 1, 2) if V != 16 else (0, 3, 2)):
+        print("conv", (Bn, H, W, C, F, R, S, stride, V, d, permute), "form", variant, flush=True)
         got = run_spconv(torch, w, R, S, C, x, stride, variant)
         assert got.shape == ref.shape
         assert not np.isnan(got.astype(np.float32)).any(), "variant %d left output elements unwritten" % variant
@@ -78,3 +79,39 @@ def test_shift_equivariance(torch_gpu):
     shifted[:, :-1, 1:] = x[:, 1:, :-1, 37]  # hi = ho + 1, wi = wo - 1
     for r in range(F):
         np.testing.assert_array_equal(got[..., w["row_permute_ids"][r]], shifted * float(w["values"][r]))
+
+
+def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
+    """The fused form keeps queues and arrival counts in its scratch and clears them when a launch ends: many
+    launches of one state in a row, with a new input each time, must all be right.  Two states over different
+    tensors own different scratch, so their launches may overlap on two streams."""
+    import shflbw_sparse_nn_amd as S
+    torch = torch_gpu
+    Bn, H, W, C, F, R, Sx, stride, V = 8, 14, 14, 64, 256, 3, 3, 1, 64
+    w = P.make_weight(F, R * Sx * C, V, 0.2, True, 2021, integer=True)
+    f = P.upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
+    rng = np.random.default_rng(31)
+    xs = [rng.integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16) for _ in range(3)]
+    refs = [O.float_to_half(P.conv_oracle(w, R, Sx, C, x, stride)) for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    dX = [torch.empty((Bn, H, W, C), dtype=torch.float16, device="cuda") for _ in range(2)]
+    dY = [torch.empty(refs[0].shape, dtype=torch.float16, device="cuda") for _ in range(2)]
+    ops = []
+    for i in range(2):
+        op = S.SpconvBlockwiseOp(3)
+        op.initialize(f, Bn, H, W, stride, dX[i].data_ptr(), dY[i].data_ptr())
+        ops.append(op)
+    assert ops[0]._state.planes != ops[1]._state.planes  # scratch is per (geometry, tensors)
+    for rnd in range(6):
+        print("fused conv round", rnd, flush=True)
+        for i in range(2):
+            dX[i].copy_(P.to_dev(torch, xs[(rnd + i) % 3]))
+            dY[i].fill_(float("nan"))
+        torch.cuda.synchronize()
+        for i in range(2):
+            for _ in range(3):  # back to back on its stream, overlapping the other stream's launches
+                ops[i](streams[i].cuda_stream)
+        torch.cuda.synchronize()
+        for i in range(2):
+            np.testing.assert_array_equal(dY[i].cpu().numpy().view(np.uint16), refs[(rnd + i) % 3].view(np.uint16),
+                                          err_msg="round %d stream %d" % (rnd, i))
