@@ -163,6 +163,7 @@ typedef struct shflbw_spmm_state {
     const int* panel_ptr;
     int brow;
     int ldb_bytes; /* distance in bytes between two rows of B that are one kept-column id apart: N * 2 */
+    const void* zero_row; /* 1 KiB of zeros inside the library (device memory): gathered for the padding slots */
 } shflbw_spmm_state;
 
 /* C may be NULL when beta == 0.  variant < 0 selects automatically. */

@@ -161,13 +161,13 @@ static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int 
         return SHFLBW_ERR_UNSUPPORTED;
     }
     g->rows = (long)g->copies * s * s * f->C;
-    if (g->np > 0x7fffffffL || (unsigned long long)g->rows * (unsigned long long)g->pitch * 2ull > 0xffffffffull) {
+    if (g->np > 0x7fffffffL || (unsigned long long)(g->rows + 1) * (unsigned long long)g->pitch * 2ull > 0xffffffffull) {
         set_error("spconv: problem too large for the plane form (%ld rows of %ld positions)", g->rows, g->pitch);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
     g->slots = f->packed_indices.size();
-    g->planes_bytes = up256((size_t)g->rows * g->pitch * 2);
+    g->planes_bytes = up256((size_t)(g->rows + 1) * g->pitch * 2); // one more row: zeros, for the padding slots
     g->dm_bytes = up256((size_t)f->F * g->np * 2);
     g->ids_bytes = up256(g->slots * sizeof(int) + 64);
     g->Ho = (H + 2 * ph - f->R) / s + 1;
@@ -193,6 +193,7 @@ static void fill_spmm_launch_args(const shflbw_spmm_state* state, int BN, SpmmLa
     a.row_ids = state->args.A_row_indices;
     a.B = (const half_t*)state->args.B;
     a.ldb_bytes = state->ldb_bytes;
+    a.zero_row = state->zero_row;
     a.C = (const half_t*)state->args.C;
     a.D = (half_t*)state->args.D;
     a.alpha = state->args.alpha;
@@ -300,6 +301,11 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     state->panel_ptr = (const int*)w->d_group_ptr;
     state->brow = w->brow;
     state->ldb_bytes = N * 2;
+    state->zero_row = spmm_zero_row();
+    if (!state->zero_row) {
+        set_error("spmm_init: cannot look up the library's row of zeros on this device");
+        return SHFLBW_ERR_HIP;
+    }
     state->variant = variant;
     state->shared_mem_size = (size_t)v->lds_bytes;
     state->grid_dim[0] = (unsigned)(X * ((N + v->BN - 1) / v->BN));
@@ -459,7 +465,7 @@ static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, c
     state->spmm.packed_indices = (const int*)(scratch + g.planes_bytes + g.dm_bytes);
     state->spmm.packed_indices_pm = (const int*)(scratch + g.planes_bytes + g.dm_bytes + g.ids_bytes);
     state->spmm.ldb_bytes = 2;
-    state->spmm.args.K = (int)(g.rows * g.pitch); // extent of the id space
+    state->spmm.args.K = (int)((g.rows + 1) * g.pitch); // extent of the id space
     state->shared_mem_size = state->spmm.shared_mem_size; // the figures of the middle (SpMM) launch
     state->grid_dim[0] = state->spmm.grid_dim[0];
     state->block_dim[0] = state->spmm.block_dim[0];
@@ -522,6 +528,10 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
             std::vector<int> ids(slots), ids_pm(slots);
             for (size_t q = 0; q < slots; q++) {
                 const int k = f->packed_indices[q];
+                if (k < 0) { // padding slot: the row of zeros behind the last channel row
+                    ids[q] = (int)(g.rows * pitch);
+                    continue;
+                }
                 const int c = k % f->C, tap = k / f->C, r = tap / f->S, t = tap % f->S;
                 const long shift = (long)(r / s) * PW + t / s;
                 const int copy = copies == 2 ? (int)(shift & 1) : 0;
@@ -772,7 +782,8 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
     if ((rc = bind_plane_form(&st, f, g, base, false)) != SHFLBW_OK) return rc;
     hipError_t e = launch_plane_ids((const int*)f->d_packed_indices, (int*)(base + g.planes_bytes + g.dm_bytes),
                                     (int*)(base + g.planes_bytes + g.dm_bytes + g.ids_bytes), (int)g.slots, f->C, f->S,
-                                    stride, g.PW, (int)g.pitch, g.copies, (hipStream_t)stream);
+                                    stride, g.PW, (int)g.pitch, g.copies, (int)(g.rows * g.pitch), (half_t*)base,
+                                    (hipStream_t)stream);
     if (e != hipSuccess) {
         set_error("spconv_exec_static: id launch failed: %s", hipGetErrorString(e));
         return SHFLBW_ERR_HIP;

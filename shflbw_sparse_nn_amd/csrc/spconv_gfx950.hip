@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const int hi = (pix_hw[e] >> 16) - 0x4000 + r, wi = (pix_hw[e] & 0xffff) - 0x4000 + s;
-                const bool ok = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                const bool ok = k >= 0 && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W; // k < 0: padding slot
                 piece[j][e] = ok ? a.in[pix_base[e] + tap] : (half_t)0.f;
             }
         }
@@ -657,27 +657,32 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_fused_kernel(Spmm
 // the rewrite shflbw_spconv_init does on the host.
 __global__ void __launch_bounds__(256) plane_ids_kernel(const int* __restrict__ kidx, int* __restrict__ ids,
                                                         int* __restrict__ ids_pm, int slots, int C, int S, int stride,
-                                                        int PW, int pitch, int copies)
+                                                        int PW, int pitch, int copies, int zero_id, half_t* planes)
 {
     const int q = blockIdx.x * 256 + threadIdx.x;
+    // the row of zeros behind the last channel row, which the padding slots gather
+    for (int i = q * 8; i < pitch; i += gridDim.x * 256 * 8) *(half8_t*)(planes + (size_t)zero_id + i) = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     if (q >= slots) return;
     const int k = kidx[q];
-    const int c = k % C, tap = k / C, r = tap / S, t = tap % S;
-    const int shift = (r / stride) * PW + t / stride;
-    const int copy = copies == 2 ? (shift & 1) : 0;
-    const int phase = (r % stride) * stride + t % stride;
-    const int id = ((copy * stride * stride + phase) * C + c) * pitch + shift - copy;
+    int id = zero_id; // padding slot
+    if (k >= 0) {
+        const int c = k % C, tap = k / C, r = tap / S, t = tap % S;
+        const int shift = (r / stride) * PW + t / stride;
+        const int copy = copies == 2 ? (shift & 1) : 0;
+        const int phase = (r % stride) * stride + t % stride;
+        id = ((copy * stride * stride + phase) * C + c) * pitch + shift - copy;
+    }
     ids[q] = id;
     const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, rr = q % 4;
     ids_pm[grp * 64 + 16 * p + 4 * j + rr] = id;
 }
 
 hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, int C, int S, int stride, int PW,
-                            int pitch, int copies, hipStream_t stream)
+                            int pitch, int copies, int zero_id, half_t* planes, hipStream_t stream)
 {
     if (slots <= 0) return hipSuccess;
     hipLaunchKernelGGL(plane_ids_kernel, dim3((slots + 255) / 256), dim3(256), 0, stream, kidx, ids, ids_pm, slots, C, S,
-                       stride, PW, pitch, copies);
+                       stride, PW, pitch, copies, zero_id, planes);
     return hipGetLastError();
 }
 

@@ -88,9 +88,10 @@ hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, i
                                  hipStream_t stream);
 
 // Plane-form ids computed on the device (for callers that may not copy from the host): slot-ordered and
-// producer-major element offsets from the packed kept-column ids.
+// producer-major element offsets from the packed kept-column ids; padding slots get `zero_id`, the offset of a
+// row of `pitch` zeros in `planes`, which the same launch clears.
 hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, int C, int S, int stride, int PW,
-                            int pitch, int copies, hipStream_t stream);
+                            int pitch, int copies, int zero_id, half_t* planes, hipStream_t stream);
 
 // Stages 1 and 3 of the im2col form of the convolution: NHWC input -> im2col matrix with rows of NP
 // halves (NP a multiple of 64), and filter-major result -> NHWC output.

@@ -16,6 +16,7 @@
 //    the vector-memory counter only ever counts the LDS copies and the waits are exact;
 //  * fp32 accumulators are rounded once to fp16, staged through LDS and scattered as whole
 //    row segments through the permutation.
+#include <mutex>
 #include <type_traits>
 
 #include "kernel_common.h"
@@ -139,8 +140,10 @@ __global__ void __launch_bounds__(NWAVES * 64) spmm_shflbw_kernel(SpmmLaunchArgs
             int k = ks[j * RPI];
 #pragma unroll
             for (int q = 1; q < RPI; q++) k = (sub == q) ? ks[j * RPI + q] : k;
-            global_to_lds_16B((const half_t*)((const char*)a.B + (size_t)k * a.ldb_bytes) + gcol[j],
-                              sb + (wave * IPW + j) * 1024);
+            // a padding slot (id -1) gathers 16 bytes per lane of the row of zeros
+            const half_t* src = k < 0 ? (const half_t*)a.zero_row + lane * 8
+                                      : (const half_t*)((const char*)a.B + (size_t)k * a.ldb_bytes) + gcol[j];
+            global_to_lds_16B(src, sb + (wave * IPW + j) * 1024);
         }
     };
 
@@ -255,7 +258,9 @@ __device__ __forceinline__ int ks_sel(const int (&ks)[N_], int base, int sub, in
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
-__global__ void __launch_bounds__((NCONS + NPROD) * 64) spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
+__global__ void
+__launch_bounds__((NCONS + NPROD) * 64, (SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>::WGS_PER_CU * (NCONS + NPROD) + 3) / 4)
+spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
 
@@ -296,7 +301,7 @@ static hipError_t launch_ws(const SpmmLaunchArgs& a, hipStream_t stream)
     if ((unsigned long long)a.K * (unsigned long long)a.ldb_bytes + (unsigned long long)a.N * 2ull > 0xffffffffull)
         return hipErrorInvalidValue;
     // one persistent workgroup per compute unit; fewer when there are fewer tiles (multiple of 8 XCDs)
-    int grid = a.num_cus > 0 ? a.num_cus : 256;
+    int grid = (a.num_cus > 0 ? a.num_cus : 256) * Cfg::WGS_PER_CU;
     grid = (grid / 8) * 8;
     const int need = ((T + 7) / 8) * 8;
     if (grid > need) grid = need;
@@ -358,6 +363,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_WS_VARIANT(64, 64, 8, 8, 32, 4),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 32, 3),
     SHFLBW_WS_VARIANT(64, 128, 4, 4, 16, 4),
+    SHFLBW_WS_VARIANT(64, 64, 4, 4, 32, 3), // two workgroups per compute unit
     SHFLBW_VARIANT(64, 64, 4, 32, 3),
     SHFLBW_VARIANT(64, 64, 4, 32, 2),
     SHFLBW_VARIANT(64, 64, 4, 16, 4),
@@ -369,6 +375,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
     SHFLBW_WS_VARIANT(32, 64, 4, 4, 32, 6),
+    SHFLBW_WS_VARIANT(32, 64, 4, 4, 32, 3), // two workgroups per compute unit
     SHFLBW_VARIANT(32, 64, 4, 32, 3),
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
@@ -381,6 +388,25 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(128, 64, 4, 32, 3),
     SHFLBW_VARIANT(128, 32, 4, 32, 3),
 };
+
+// The row of zeros the padding slots gather.  `g_zero_row` is the host-side handle of the symbol; kernels get
+// the device address, looked up once per device.
+static __device__ __align__(1024) unsigned char g_zero_row[1024];
+
+const void* spmm_zero_row()
+{
+    static std::mutex lock;
+    static void* addr[64] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!addr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_zero_row)) != hipSuccess) return nullptr;
+        addr[dev] = p;
+    }
+    return addr[dev];
+}
 
 const SpmmVariant* spmm_variants(int* count)
 {

@@ -15,6 +15,7 @@ struct SpmmLaunchArgs {
     const int* panel_desc;  // private image: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
     const int* row_ids;     // M, or null when rows are not permuted
     const half_t* B;
+    const void* zero_row;   // 1 KiB of zeros on the device: what the padding slots (id -1) of a panel's last group gather
     int ldb_bytes;          // bytes between rows of B one id apart (N * 2 for a dense row-major B)
     const half_t* C;
     half_t* D;
@@ -37,5 +38,8 @@ struct SpmmVariant {
 };
 
 const SpmmVariant* spmm_variants(int* count);
+
+// device address of the library's row of zeros on the current device (looked up once per device); null on failure
+const void* spmm_zero_row();
 
 } // namespace shflbw

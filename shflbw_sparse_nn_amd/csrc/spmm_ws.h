@@ -56,6 +56,9 @@ struct SpmmWsCfg {
     static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int LDS_BYTES = RING_BYTES + NCONS * EPI_WAVE_BYTES;
     static constexpr int THREADS = (NCONS + NPROD) * 64;
+    // Workgroups a compute unit holds at once.  Two of them (their rings together fill the LDS, their registers
+    // the file: at most 128 per wave) let one workgroup's epilogue stores run beside the other's stage loop.
+    static constexpr int WGS_PER_CU = LDS_BYTES <= 79 * 1024 && THREADS <= 512 ? 2 : 1;
     static_assert((V % 32 == 0 || (V == 16 && KT == 32)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
     static_assert(BN == 512 || (BN == 256 && RPW == 8), "a 1 KiB copy instruction covers one gathered row, or two");
     static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
@@ -569,9 +572,14 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
     uint32_t va = 0;             // lane offset of this wave's A fragment of the next stage
     uint32_t dva = 0;            // ... and its step from stage to stage
     const char* tileA = nullptr; // A fragments of the current tile
+    // Padding slots (id -1, only in the last group of a panel) gather from the row of zeros: its address less the
+    // tile's column offset, so that the lane offsets voff[] of the tile apply to it as they do to a row of B.
+    const char* zb = nullptr;
+    bool pad_group = false;      // the group being issued may hold padding slots
     auto open_tile = [&]() __attribute__((always_inline)) {
         const int n0 = (id / X) * BN;
         tileA = (const char*)a.packedA + (size_t)cur.y * (64 * V * 2);
+        zb = (const char*)a.zero_row - (size_t)n0 * 2;
         const int nst = (cur.x + KSPS - 1) / KSPS;
         va = pw * 1024 + lane * 16 + (rev ? (uint32_t)(nst - 1) * (Cfg::A_FRAGS * 1024) : 0u);
         dva = rev ? (uint32_t) - (Cfg::A_FRAGS * 1024) : (uint32_t)(Cfg::A_FRAGS * 1024);
@@ -583,7 +591,7 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
             const int pc = Cfg::RPI == 1 ? lane : lane & 31;
             const int lc = ((((pc >> 1) ^ row_xor32(key))) << 1) | (pc & 1);
             const int col = n0 + lc * 8;
-            int c = col < N ? col : 0; // columns past N are never stored
+            int c = col < N ? col : n0; // columns past N are never stored; any valid column of the tile will do
             if (CONV) c += (c / a.img_cols) * a.img_skip;
             voff[j] = (uint32_t)c * 2;
         }
@@ -606,7 +614,36 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
         auto stage = [&](int4_t ka, int4_t kb) __attribute__((always_inline)) {
             __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * MYOPS));
             wg_barrier();
-            if (Cfg::RPI == 1) {
+            if (pad_group) {
+                // same copies, one at a time, each from B or from the row of zeros
+                const int ks[8] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
+                if (Cfg::RPI == 1) {
+                    auto row = [&](auto jj) __attribute__((always_inline)) {
+                        constexpr int j = decltype(jj)::value;
+                        const bool pad = ks[j] < 0;
+                        global_to_lds_16B_sbase<j * 0x400>(pad ? (const void*)zb : (const void*)a.B,
+                                                           (pad ? 0u : (uint32_t)ks[j] * rowbytes) + voff[j & 3], sbp);
+                    };
+                    row(std::integral_constant<int, 0>{});
+                    row(std::integral_constant<int, 1>{});
+                    row(std::integral_constant<int, 2>{});
+                    row(std::integral_constant<int, 3>{});
+                    if (RPW == 8) {
+                        row(std::integral_constant<int, 4>{});
+                        row(std::integral_constant<int, 5>{});
+                        row(std::integral_constant<int, 6>{});
+                        row(std::integral_constant<int, 7>{});
+                    }
+                } else {
+                    const bool hi = lane >= 32;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int k = hi ? ks[2 * j + 1] : ks[2 * j];
+                        const char* src = k < 0 ? zb : (const char*)a.B + (size_t)((uint32_t)k * rowbytes);
+                        global_to_lds_16B(src + voff[j], sbp + j * 0x400);
+                    }
+                }
+            } else if (Cfg::RPI == 1) {
                 gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
                 if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
             } else {
@@ -709,6 +746,7 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
                     gnext = nxt.x > 0 ? nxt.y + ((rev != (a.alternate != 0)) ? groups_of(nxt.x) - 1 : 0) : cur.y + g;
                 const int4_t gn0 = *group_ptr(gnext, 0), gn1 = *group_ptr(gnext, 1), gn2 = *group_ptr(gnext, 2),
                              gn3 = *group_ptr(gnext, 3);
+                pad_group = g + 1 == ngroups;
                 issue_group(n, rev);
                 if (!have_next) { // deferred from the start: not needed before the first copies are out
                     find_next();

@@ -195,8 +195,8 @@ static int check_pattern(int nrow, int ncol, int brow, int bcol, int nnzb, const
 
 // ---------------------------------------------------------------------------------
 // private image.  Panel i keeps nnz_i vectors; they are padded to a multiple of 64
-// slots.  packed_indices: the column ids, tail slots repeat the last valid id (their
-// values are zero).  packed_values: per MFMA k-step, the A operand in register
+// slots.  packed_indices: the column ids, tail slots hold -1 (their values are zero and
+// the kernels gather a row of zeros for them, so that a non-finite B cannot leak through 0 * x).  packed_values: per MFMA k-step, the A operand in register
 // order, so one wave reads a fragment as 64 consecutive 16-byte pieces:
 //   V >= 32 (32x32x16 tiles): step s covers slots 16s..16s+15; block mb covers rows
 //     32mb..32mb+31; lane l holds row 32mb + l%32, slots 16s + 8*(l/32) + 0..7.
@@ -234,7 +234,7 @@ int build_packed_image(shflbw_weight* w)
         const size_t slot0 = (size_t)w->group_ptr[i] * 64;
         const int padded = (w->group_ptr[i + 1] - w->group_ptr[i]) * 64;
         for (int q = 0; q < padded; q++)
-            w->packed_indices[slot0 + q] = w->indices[begin + std::min(q, nnz - 1)];
+            w->packed_indices[slot0 + q] = q < nnz ? w->indices[begin + q] : -1; // padding: gathered from a row of zeros
         for (int q = 0; q < padded; q++) {
             const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, r = q % 4;
             w->packed_indices_pm[slot0 + grp * 64 + 16 * p + 4 * j + r] = w->packed_indices[slot0 + q];

@@ -26,7 +26,7 @@ struct shflbw_weight {
     // private image for the gfx950 kernels, built by sync_device
     std::vector<int> group_ptr;      // X+1: cumulative count of 64-slot groups per panel
     std::vector<int> panel_desc;     // 2X: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
-    std::vector<int> packed_indices; // 64 * group_ptr[X]; tail slots repeat the panel's last id
+    std::vector<int> packed_indices; // 64 * group_ptr[X]; tail slots hold -1 (a row of zeros)
     std::vector<int> packed_indices_pm; // each 64-slot group reordered: [16p + 4j + r] = packed_indices[16j + 4p + r]
     std::vector<uint16_t> packed_values; // 64 * brow * group_ptr[X]; MFMA fragment order, tail zero
 

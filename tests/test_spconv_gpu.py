@@ -115,3 +115,24 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
         for i in range(2):
             np.testing.assert_array_equal(dY[i].cpu().numpy().view(np.uint16), refs[(rnd + i) % 3].view(np.uint16),
                                           err_msg="round %d stream %d" % (rnd, i))
+
+
+def test_non_finite_input_does_not_leak_through_padding(torch_gpu):
+    """Padding slots of the filter's panels gather zeros (a row of zeros behind the planes, a row of zeros in the
+    library for the im2col form, nothing in the direct kernel): an Inf in the input reaches only the outputs
+    whose kept taps read it."""
+    Bn, H, W, C, F, R, Sx, stride, V = 2, 9, 10, 16, 64, 3, 3, 1, 32
+    w = P.make_weight(F, R * Sx * C, V, 0.3, True, 5, integer=True)
+    w["values"] = np.where(w["values"] == 0, np.float16(1), w["values"]).astype(np.float16)
+    x = np.random.default_rng(6).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
+    x[0, 4, 5, 3] = np.inf
+    x[1, 0, 0, C - 1] = -np.inf
+    x[1, 8, 9, 7] = np.nan
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = O.float_to_half(P.conv_oracle(w, R, Sx, C, x, stride))
+    assert np.isfinite(ref.astype(np.float32)).any() and not np.isfinite(ref.astype(np.float32)).all()
+    for variant in (0, 1, 2, 3):
+        got = run_spconv(torch_gpu, w, R, Sx, C, x, stride, variant)
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), "form %d: NaN pattern differs" % variant
+        ok = ~np.isnan(ref)
+        np.testing.assert_array_equal(got[ok], ref[ok], err_msg="form %d" % variant)

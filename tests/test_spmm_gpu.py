@@ -146,3 +146,25 @@ def test_linearity_full_size(torch_gpu):
     d2 = run_spmm(torch_gpu, w, B2).astype(np.float32)
     d12 = run_spmm(torch_gpu, w, (B1 + B2).astype(np.float16)).astype(np.float32)
     np.testing.assert_array_equal(d12, d1 + d2)
+
+
+@pytest.mark.parametrize("V", [16, 32, 64, 128])
+def test_non_finite_activations_do_not_leak_through_padding(torch_gpu, V):
+    """A panel's kept vectors are padded to whole groups of 64 slots with zero weights.  The padding gathers a row
+    of zeros, not a row of B, so an Inf or NaN in B reaches exactly the outputs it reaches in the reference: rows
+    of panels that keep that column.  Every tile variant; panel sizes that leave 1 .. 63 padding slots."""
+    M, K, N = 4 * V, 192, 520
+    w = P.make_weight(M, K, V, 0.3, True, 77, integer=True)
+    w["values"] = np.where(w["values"] == 0, np.float16(1), w["values"]).astype(np.float16)  # 0 * inf is NaN in the reference too
+    B = P.make_dense(K, N, 78, integer=True).astype(np.float16)
+    B[5, :] = np.inf
+    B[77, 3::7] = -np.inf
+    B[130, 1::5] = np.nan
+    B[K - 1, :] = np.inf  # the largest column id: what a repeated last id would have hit
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = O.float_to_half(P.spmm_oracle(w, B))
+    for variant in range(len(S.spmm_variants(V))):
+        got = run_spmm(torch_gpu, w, B, variant=variant)
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), "variant %d: NaN pattern differs" % variant
+        ok = ~np.isnan(ref)
+        np.testing.assert_array_equal(got[ok], ref[ok], err_msg="variant %d" % variant)
