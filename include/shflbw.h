@@ -114,6 +114,10 @@ int shflbw_spmm_host_reference(const shflbw_weight* w, int N, const uint16_t* B,
                                const uint16_t* C, float beta, float* D_ref);
 int shflbw_spconv_host_reference(const shflbw_weight* filter, int B, int H, int W, int stride,
                                  const uint16_t* IFMap, float* OFMap_ref);
+/* ... and over the reference's C-H-W-B / F-H-W-B tensors with its own bounds rule (see shflbw_spconv_init_chwb):
+ * spconv/blockwise_format.h:55-132 as it stands. */
+int shflbw_spconv_host_reference_chwb(const shflbw_weight* filter, int B, int H, int W, int stride,
+                                      const uint16_t* IFMap, float* OFMap_ref);
 
 int shflbw_weight_get_info(const shflbw_weight* w, shflbw_weight_info* info);
 /* Borrowed pointers to the host arrays (valid until the weight is re-initialised/destroyed). */
@@ -240,6 +244,14 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* filter,
 int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* filter,
                                int B, int H, int W, int stride, const void* IFMap, void* OFMap, int variant);
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream);
+/* The same operator over the reference's own tensors (spconv/blockwise_format.h:111-128, spconv/conv_format.h:49-82):
+ * IFMap[c][hi][wi][b] and OFMap[f][ho][wo][b], batch innermost; H and W are the extents of the output grid and at
+ * the same time the bounds of the input: out(ho, wo) reads in(ho*stride - R/2 + r, wo*stride - S/2 + s) where that lies
+ * inside H x W and zero elsewhere (so IFMap holds C*H*W*B values and OFMap F*H*W*B, whatever the stride).
+ * Precondition as in the reference's kernel (spconv/blockwise_kernel.h:200-207): B % 8 == 0.  exec launches a padded
+ * copy of the input and one SpMM launch that writes OFMap directly (form 4 of shflbw_spconv_variant_name). */
+int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* filter,
+                            int B, int H, int W, int stride, const void* IFMap, void* OFMap);
 /* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  One complete convolution in the plane
  * form, the same launches as shflbw_spconv_init + shflbw_spconv_exec, with all scratch (the planes, the

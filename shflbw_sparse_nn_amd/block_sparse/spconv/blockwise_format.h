@@ -9,8 +9,18 @@ enum LayoutFilter {
     filter_planar_first   // F-C-R-S
 };
 
+// Layout of the feature maps the operators of a filter work on.  fmap_nhwc (the default here): IFMap[b][hi][wi][c],
+// OFMap[b][ho][wo][f], H and W the input extents, true stride.  fmap_batch_first: the reference's own tensors,
+// IFMap[c][h][w][b] and OFMap[f][h][w][b] with H, W bounding input and output alike
+// (spconv/blockwise_format.h:111-128); set `spfilter.fmap_layout = fmap_batch_first;` before initialize().
+enum LayoutFmap {
+    fmap_nhwc,
+    fmap_batch_first
+};
+
 template <typename T>
 struct BlockwiseSpFilter : public BlockwiseSpMatrix<T> {
+    LayoutFmap fmap_layout = fmap_nhwc;
     int F = 0; // filters (output channels)
     int C = 0; // input channels
     int R = 0; // filter rows
@@ -32,9 +42,10 @@ struct BlockwiseSpFilter : public BlockwiseSpMatrix<T> {
                                    LayoutFilter layout_filter);
 };
 
-// The convolution on the CPU, fp32 (spconv/blockwise_format.h:55-132), over this library's tensors: NHWC,
-// H and W are the input extents, padding R/2 and S/2, output [B][Ho][Wo][F] with
-// Ho = (H + 2*(R/2) - R)/stride + 1.  Only filter_channel_first filters exist here.
+// The convolution on the CPU, fp32 (spconv/blockwise_format.h:55-132), over the tensors `spfilter.fmap_layout`
+// names: NHWC with H and W the input extents, padding R/2 and S/2, output [B][Ho][Wo][F] with
+// Ho = (H + 2*(R/2) - R)/stride + 1; or, for fmap_batch_first, the reference's C-H-W-B input and F-H-W-B output of
+// B*H*W*F values.  Only filter_channel_first filters exist here.
 template <typename T>
 void get_host_reference(BlockwiseSpFilter<T>& spfilter, const int B, const int H, const int W, const int stride,
                         const std::vector<T>& IFMap, std::vector<float>& OFMap_ref,
@@ -43,6 +54,12 @@ void get_host_reference(BlockwiseSpFilter<T>& spfilter, const int B, const int H
     assert(layout_filter == filter_channel_first);
     (void)layout_filter;
     spfilter.push_host_arrays();
+    if (spfilter.fmap_layout == fmap_batch_first) {
+        OFMap_ref.resize(static_cast<size_t>(B) * H * W * spfilter.F);
+        SHFLBW_CHECK(shflbw_spconv_host_reference_chwb(spfilter.handle(), B, H, W, stride,
+                                                       reinterpret_cast<const uint16_t*>(IFMap.data()), OFMap_ref.data()));
+        return;
+    }
     const int Ho = (H + 2 * (spfilter.R / 2) - spfilter.R) / stride + 1;
     const int Wo = (W + 2 * (spfilter.S / 2) - spfilter.S) / stride + 1;
     OFMap_ref.resize(static_cast<size_t>(B) * Ho * Wo * spfilter.F);

@@ -2,12 +2,13 @@
 // SpconvBlockwiseInitFn / ExecFn and their pointer types (block_sparse/spconv/blockwise_op.h:6-17,
 // 19-149, 161-193), forwarding to shflbw_spconv_init / shflbw_spconv_exec.
 //
-// Tensor layout differs from the reference on purpose: feature maps are NHWC
+// Tensor layout differs from the reference by default: feature maps are NHWC
 // (IFMap[b][hi][wi][c], OFMap[b][ho][wo][f]), H and W are the input extents, and stride is a
 // true stride (output extent (H + 2*(R/2) - R)/stride + 1); the reference's maps are
 // C-H-W-B / F-H-W-B with H, W doubling as input and output extent
 // (spconv/blockwise_format.h:111-128).  The implicit-GEMM view (M = F, K ordered (r, s, c),
-// zero for out-of-bounds taps, row permutation on F) is the reference's.
+// zero for out-of-bounds taps, row permutation on F) is the reference's.  A filter whose fmap_layout is
+// fmap_batch_first gets the reference's own tensors and bounds rule instead.
 #pragma once
 #include "blockwise_format.h"
 
@@ -34,7 +35,9 @@ inline SpconvBlockwiseOpState spconv_make_state(BlockwiseSpFilter<half>& spfilte
     assert(spfilter.brow == block_height && "operator block height must equal the filter block height");
     assert(spfilter.bcol == 1);
     assert(spfilter.device_synced);
-    int rc = shflbw_spconv_init(&st.native, spfilter.handle(), B, H, W, stride, IFMap, OFMap);
+    int rc = spfilter.fmap_layout == fmap_batch_first
+                 ? shflbw_spconv_init_chwb(&st.native, spfilter.handle(), B, H, W, stride, IFMap, OFMap)
+                 : shflbw_spconv_init(&st.native, spfilter.handle(), B, H, W, stride, IFMap, OFMap);
     if (rc != SHFLBW_OK) {
         std::cerr << "SpconvBlockwiseOp::initialize: " << shflbw_status_string(rc) << ": " << shflbw_last_error()
                   << std::endl;

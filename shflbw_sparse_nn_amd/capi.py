@@ -23,7 +23,7 @@ EXPORTS = [
     "shflbw_spmm_init", "shflbw_spmm_init_variant", "shflbw_spmm_exec",
     "shflbw_spmm_variant_count", "shflbw_spmm_variant_name",
     "shflbw_spconv_init", "shflbw_spconv_init_variant", "shflbw_spconv_exec",
-    "shflbw_spconv_exec_static",
+    "shflbw_spconv_exec_static", "shflbw_spconv_init_chwb", "shflbw_spconv_host_reference_chwb",
     "shflbw_spconv_variant_count", "shflbw_spconv_variant_name", "shflbw_weight_release_scratch",
     "shflbw_spmm_host_reference", "shflbw_spconv_host_reference",
     "shflbw_abi_sizes", "shflbw_device_info",
@@ -122,6 +122,8 @@ def load():
     lib.shflbw_spconv_init_variant.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp, ci]
     lib.shflbw_spconv_exec.argtypes = [C.POINTER(SpconvState), vp]
     lib.shflbw_spconv_exec_static.argtypes = [vp, ci, ci, ci, ci, vp, vp, vp]
+    lib.shflbw_spconv_init_chwb.argtypes = [C.POINTER(SpconvState), vp, ci, ci, ci, ci, vp, vp]
+    lib.shflbw_spconv_host_reference_chwb.argtypes = [vp, ci, ci, ci, ci, vp, vp]
     lib.shflbw_spconv_variant_count.argtypes = []
     lib.shflbw_spconv_variant_name.restype = C.c_char_p
     lib.shflbw_spconv_variant_name.argtypes = [ci]

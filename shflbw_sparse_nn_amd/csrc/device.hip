@@ -200,6 +200,8 @@ static void fill_spmm_launch_args(const shflbw_spmm_state* state, int BN, SpmmLa
     a.beta = state->args.beta;
     a.num_cus = device_compute_units();
     a.img_cols = 1, a.img_skip = 0;
+    a.ldd = a.N;
+    a.dmap_row = a.dmap_valid = 0, a.dmap_magic = 0;
     a.tile_arrivals = nullptr;
     // rows of B one column tile can touch: above about 2.5 MB they do not stay in the 4 MB L2 of an XCD
     // from one round of tiles to the next, and alternating the direction of the walk pays (measured:
@@ -374,7 +376,7 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
         set_error("spconv_init: non-positive B, H, W or stride");
         return SHFLBW_ERR_INVALID;
     }
-    if ((f->C % 8) != 0 || (f->F % 8) != 0) {
+    if (variant != 4 && ((f->C % 8) != 0 || (f->F % 8) != 0)) { // NHWC forms move 8 channels / 8 filters at a time
         set_error("spconv_init: C and F must be multiples of 8 (got %d, %d)", f->C, f->F);
         return SHFLBW_ERR_SHAPE;
     }
@@ -478,6 +480,11 @@ static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, c
 int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
                                const void* IFMap, void* OFMap, int variant)
 {
+    if (variant == 4) {
+        if (state) memset(state, 0, sizeof(*state));
+        set_error("spconv_init: form 4 works on C-H-W-B / F-H-W-B tensors; call shflbw_spconv_init_chwb");
+        return SHFLBW_ERR_INVALID;
+    }
     int frc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
     if (frc != SHFLBW_OK) return frc;
     const int Ho = state->Ho, Wo = state->Wo;
@@ -584,6 +591,95 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     return SHFLBW_OK;
 }
 
+int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                            const void* IFMap, void* OFMap)
+{
+    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, 4);
+    if (rc != SHFLBW_OK) return rc;
+    if (B % 8 != 0) { // the reference's kernel moves 8 batch entries at a time (spconv/blockwise_kernel.h:200-207)
+        set_error("spconv_init_chwb: the batch must be a multiple of 8 (got %d)", B);
+        return SHFLBW_ERR_SHAPE;
+    }
+    const ConvChwbKernel* k = conv_chwb_kernel(f->brow);
+    if (!k) {
+        set_error("spconv_init_chwb: no kernel for block size %d", f->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    SHFLBW_HIP_TRY(k->prepare());
+    // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
+    state->Ho = H;
+    state->Wo = W;
+    const int s = stride;
+    const long PHX = H + (f->R - 1) / s, PW = W + (f->S - 1) / s;
+    const long np = PHX * PW * B;                                  // values of one channel plane
+    const long pitch = (np + (long)((f->S - 1) / s) * B + 8 + 63) / 64 * 64;
+    const long rows = (long)s * s * f->C;
+    const long ncols = (long)H * PW * B;                           // columns of the GEMM: the padded output grid
+    if (ncols > 0x7fffffffL || (unsigned long long)(rows + 1) * (unsigned long long)pitch * 2ull > 0xffffffffull) {
+        set_error("spconv_init_chwb: problem too large (%ld channel rows of %ld values)", rows, pitch);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
+    const size_t slots = f->packed_indices.size();
+    const size_t planes_bytes = up256((size_t)(rows + 1) * pitch * 2), ids_bytes = up256(slots * sizeof(int) + 64);
+    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is bookkeeping of the handle (see shflbw_spconv_init_variant)
+    std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
+    char* scratch = nullptr;
+    const int key[5] = {4, B, H, W, stride};
+    for (auto& sc : fw->conv_scratch)
+        if (sc.bytes == planes_bytes + 2 * ids_bytes && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap)
+            scratch = (char*)sc.ptr;
+    if (!scratch) {
+        void* ptr = nullptr;
+        if (hipMalloc(&ptr, planes_bytes + 2 * ids_bytes) != hipSuccess) {
+            set_error("spconv_init_chwb: cannot allocate %zu bytes of device scratch", planes_bytes + 2 * ids_bytes);
+            return SHFLBW_ERR_HIP;
+        }
+        fw->conv_scratch.push_back(shflbw_weight::Scratch{planes_bytes + 2 * ids_bytes, ptr, {4, B, H, W, stride}, IFMap, OFMap});
+        scratch = (char*)ptr;
+        SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes)); // includes the row of zeros behind the last channel row
+        // kept-column id k = (r*S + t)*C + c  ->  element offset of the (phase, channel) row + tap offset
+        std::vector<int> ids(slots), ids_pm(slots);
+        for (size_t q = 0; q < slots; q++) {
+            const int kk = f->packed_indices[q];
+            if (kk < 0) {
+                ids[q] = (int)(rows * pitch);
+                continue;
+            }
+            const int c = kk % f->C, tap = kk / f->C, r = tap / f->S, t = tap % f->S;
+            ids[q] = (int)((((long)(r % s) * s + t % s) * f->C + c) * pitch + ((long)(r / s) * PW + t / s) * B);
+        }
+        for (size_t q = 0; q < slots; q++) { // producer-major order inside every 64-slot group
+            const size_t grp = q / 64;
+            const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
+            ids_pm[grp * 64 + 16 * p + 4 * j + r] = ids[q];
+        }
+        SHFLBW_HIP_TRY(hipMemcpy(scratch + planes_bytes, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+        SHFLBW_HIP_TRY(hipMemcpy(scratch + planes_bytes + ids_bytes, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+    }
+    state->planes = scratch;
+    state->np = (int)np;
+    state->plane_rows = (int)PHX;
+    state->plane_cols = (int)PW;
+    state->plane_pitch = (int)pitch;
+    state->plane_copies = 1;
+    state->ncols = (int)ncols;
+    // the SpMM in the middle writes the output tensor itself: row f of the result is the F-H-W-B row of filter f
+    rc = shflbw_spmm_init_variant(&state->spmm, f, (int)ncols, state->planes, nullptr, OFMap, 1.f, 0.f, 0);
+    if (rc != SHFLBW_OK) return rc;
+    state->spmm.packed_indices = (const int*)(scratch + planes_bytes);
+    state->spmm.packed_indices_pm = (const int*)(scratch + planes_bytes + ids_bytes);
+    state->spmm.ldb_bytes = 2;
+    state->spmm.args.K = (int)((rows + 1) * pitch);
+    state->shared_mem_size = (size_t)k->lds_bytes;
+    state->grid_dim[0] = (unsigned)((f->nrow / f->brow) * ((ncols + k->BN - 1) / k->BN));
+    state->block_dim[0] = (unsigned)k->threads;
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
 {
     if (!state || !state->init_success) {
@@ -613,6 +709,25 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
+    if (state->variant == 4) {
+        const ConvChwbKernel* k = conv_chwb_kernel(state->brow);
+        if (!k) return SHFLBW_ERR_UNSUPPORTED;
+        hipError_t e = launch_chwb_to_planes(a.in, (half_t*)state->planes, a.B, a.H, a.W, a.C, a.R, a.S, a.stride,
+                                             state->plane_rows, state->plane_cols, state->plane_pitch, (hipStream_t)stream);
+        SpmmLaunchArgs m;
+        fill_spmm_launch_args(&state->spmm, k->BN, &m);
+        m.alternate = 0;
+        m.ldd = a.H * a.W * a.B;                    // a row of the output: one filter, H x W x B values
+        m.dmap_row = state->plane_cols * a.B;       // columns of the GEMM per row of the padded output grid
+        m.dmap_valid = a.W * a.B;                   // ... of which the first W x B are output values
+        m.dmap_magic = udiv_magic(m.dmap_row);
+        if (e == hipSuccess && m.X > 0) e = k->launch(m, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));
+            return SHFLBW_ERR_HIP;
+        }
+        return SHFLBW_OK;
+    }
     if (state->variant == 3) {
         const ConvFusedKernel* k = conv_fused_kernel(state->brow);
         if (!k) return SHFLBW_ERR_UNSUPPORTED;
@@ -796,6 +911,7 @@ static const char* const g_spconv_forms[] = {
     "direct",                 // 1: one kernel, im2col gather from NHWC in the tile loads
     "im2col+spmm+transpose",  // 2: explicit im2col matrix, three launches
     "fused-planes",           // 3: the steps of form 0 in one persistent launch
+    "chwb-planes+spmm",       // 4: the reference's batch-innermost tensors (shflbw_spconv_init_chwb only): padded copy, SpMM
 };
 
 int shflbw_spconv_variant_count(void) { return (int)(sizeof(g_spconv_forms) / sizeof(g_spconv_forms[0])); }

@@ -113,4 +113,43 @@ int shflbw_spconv_host_reference(const shflbw_weight* f, int B, int H, int W, in
     return SHFLBW_OK;
 }
 
+int shflbw_spconv_host_reference_chwb(const shflbw_weight* f, int B, int H, int W, int stride, const uint16_t* IFMap,
+                                      float* OFMap_ref)
+{
+    int rc = usable(f, "spconv_host_reference_chwb");
+    if (rc) return rc;
+    if (f->R <= 0) {
+        set_error("spconv_host_reference_chwb: weight has no filter view");
+        return SHFLBW_ERR_STATE;
+    }
+    if (B <= 0 || H <= 0 || W <= 0 || stride <= 0 || !IFMap || !OFMap_ref) {
+        set_error("spconv_host_reference_chwb: null tensor or non-positive extent");
+        return SHFLBW_ERR_INVALID;
+    }
+    // tensors C-H-W-B and F-H-W-B; H, W bound input and output alike (spconv/blockwise_format.h:111-128)
+    const int V = f->brow, X = f->F / V, Cc = f->C, R = f->R, S = f->S;
+    const size_t plane = (size_t)H * W * B;
+    const std::vector<float> in = widen(IFMap, plane * Cc);
+    memset(OFMap_ref, 0, sizeof(float) * plane * f->F);
+    for (int panel = 0; panel < X; panel++)
+        for (int p = f->indptr[panel]; p < f->indptr[panel + 1]; p++) {
+            const int k = f->indices[p], c = k % Cc, tap = k / Cc, t = tap % S, rr = tap / S;
+            for (int r = 0; r < V; r++) {
+                const int stored = panel * V + r;
+                const float wv = half_to_float(f->values[(size_t)p * V + r]);
+                float* out = OFMap_ref + (size_t)(f->row_permute ? f->row_permute_ids[stored] : stored) * plane;
+                for (int ho = 0; ho < H; ho++) {
+                    const int hi = ho * stride - R / 2 + rr;
+                    if (hi < 0 || hi >= H) continue;
+                    for (int wo = 0; wo < W; wo++) {
+                        const int wi = wo * stride - S / 2 + t;
+                        if (wi < 0 || wi >= W) continue;
+                        axpy(wv, in.data() + ((size_t)(c * H + hi) * W + wi) * B, out + ((size_t)ho * W + wo) * B, B);
+                    }
+                }
+            }
+        }
+    return SHFLBW_OK;
+}
+
 } // extern "C"

@@ -98,6 +98,22 @@ __device__ __forceinline__ void store_result_16B(half_t* p, half8_t v)
 // one line are served one after the other (about 11 ns each with every compute unit taking part).
 constexpr int SYNC_LINE = 64; // ints
 
+// n / d and n % d for n < 2^31 with magic = floor(2^32 / d) computed on the host (udiv_magic below): the product's high word
+// is the quotient or one less, one correction step settles it; an integer division by a run-time value costs about
+// forty instructions, and the layout phases do several per 16-byte piece
+__device__ __forceinline__ void fast_divmod(int n, int d, unsigned magic, int& q, int& r)
+{
+    q = (int)__umulhi((unsigned)n, magic);
+    r = n - q * d;
+    if (r >= d) {
+        q++;
+        r -= d;
+    }
+}
+
+// floor(2^32 / d) for fast_divmod
+inline unsigned udiv_magic(int d) { return d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / (unsigned)d); }
+
 // Logical workgroup id for a 1-D grid: the hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs; this makes consecutive *logical* ids share an XCD (and
 // therefore its L2), so tiles that gather the same activation slab run side by side.

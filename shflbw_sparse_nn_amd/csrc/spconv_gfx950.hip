@@ -393,19 +393,6 @@ constexpr int LINE_LEFT_ALL = 0, LINE_GAVE_UP = 1, LINE_Q0 = 2, LINE_DONE0 = 10,
 #define CONV_STAMP(i) do { } while (0)
 #endif
 
-// n / d and n % d for n < 2^31 with magic = floor(2^32 / d) computed on the host (udiv_magic): the product's high word
-// is the quotient or one less, one correction step settles it; an integer division by a run-time value costs about
-// forty instructions, and the layout phases do several per 16-byte piece
-__device__ __forceinline__ void fast_divmod(int n, int d, unsigned magic, int& q, int& r)
-{
-    q = (int)__umulhi((unsigned)n, magic);
-    r = n - q * d;
-    if (r >= d) {
-        q++;
-        r -= d;
-    }
-}
-
 __device__ __forceinline__ int sync_load(const int* p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -718,6 +705,123 @@ hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int np
     const dim3 grid(NP / TT, (F + TT - 1) / TT);
     hipLaunchKernelGGL(transpose_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, npix, NP);
     return hipGetLastError();
+}
+
+// =======================================================================================
+// Convolution over the reference's own tensors (spconv/blockwise_format.h:111-128): input C-H-W-B, output
+// F-H-W-B, batch innermost, H and W the extents of the OUTPUT grid and at the same time the bounds of the input
+// (out(ho, wo) reads in(ho*stride - R/2 + r, wo*stride - S/2 + t) where that lies inside H x W, zero elsewhere).
+// With the batch innermost both ends of the GEMM are contiguous: a kept vector k = (r, t, c) is a run of channel
+// c's plane at a constant offset, and a row of the result is a row of the output.  Two launches:
+//   1. chwb_to_planes_kernel: pure copy with zero fill into padded phase planes
+//        planes[phase (a, b)][c][(i * PW + j) * B + n] = in[c][i*stride + a - R/2][j*stride + b - S/2][n]
+//      with PHX = H + (R-1)/stride rows and PW = W + (S-1)/stride columns per plane: tap (r, t) of output (ho, wo)
+//      reads phase (r % stride, t % stride) at (ho + r / stride, wo + t / stride).  B is a multiple of 8, so
+//      every tap offset is a multiple of 16 bytes and no shifted copy is needed.
+//   2. the role-split SpMM over the H * PW * B columns (ho, j, n) of the padded output grid; its epilogue maps a
+//      column to the compact output row and drops the (S-1)/stride padding columns per row (output_column()).
+// =======================================================================================
+struct ChwbGeom {
+    int B, H, W, C, stride, pad_h, pad_w;
+    int PHX, PW;  // rows and columns of a phase plane
+    int pitch;    // values per channel row of the plane tensor
+};
+
+// one thread per 16-byte piece (8 batch entries): grid.x covers the pieces of one channel plane, grid.y the channels,
+// grid.z the phases
+__global__ void __launch_bounds__(256) chwb_to_planes_kernel(const half_t* __restrict__ in, half_t* __restrict__ planes,
+                                                             ChwbGeom g, unsigned magic_row, unsigned magic_b8)
+{
+    const int b8 = g.B >> 3, row_pieces = g.PW * b8;
+    const int piece = blockIdx.x * 256 + threadIdx.x;
+    if (piece >= g.PHX * row_pieces) return;
+    const int c = blockIdx.y, phase = blockIdx.z;
+    const int pa = phase / g.stride, pb = phase % g.stride;
+    int i, rem, j, n8;
+    fast_divmod(piece, row_pieces, magic_row, i, rem);
+    fast_divmod(rem, b8, magic_b8, j, n8);
+    const int hi = i * g.stride + pa - g.pad_h, wi = j * g.stride + pb - g.pad_w;
+    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (hi >= 0 && hi < g.H && wi >= 0 && wi < g.W) v = *(const half8_t*)(in + ((size_t)(c * g.H + hi) * g.W + wi) * g.B + n8 * 8);
+    *(half8_t*)(planes + ((size_t)phase * g.C + c) * g.pitch + (size_t)piece * 8) = v;
+}
+
+hipError_t launch_chwb_to_planes(const half_t* in, half_t* planes, int B, int H, int W, int C, int R, int S, int stride,
+                                 int PHX, int PW, int pitch, hipStream_t stream)
+{
+    ChwbGeom g{B, H, W, C, stride, R / 2, S / 2, PHX, PW, pitch};
+    const int pieces = PHX * PW * (B >> 3);
+    const dim3 grid((pieces + 255) / 256, C, stride * stride);
+    hipLaunchKernelGGL(chwb_to_planes_kernel, grid, dim3(256), 0, stream, in, planes, g, udiv_magic(PW * (B >> 3)),
+                       udiv_magic(B >> 3));
+    return hipGetLastError();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+__global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_chwb_kernel(SpmmLaunchArgs a)
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // tiles as in the SpMM kernel: XCD x owns a contiguous range of the column-tile-major ids
+    const int T = a.X * a.n_tiles;
+    const int per = (T + 7) >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int S = gridDim.x >> 3;
+    const int id_first = xcd * per + (blockIdx.x >> 3);
+    const int id_end = min(T, (xcd + 1) * per);
+    if (wave >= NCONS)
+        ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE, false>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
+    else if constexpr (V == 16)
+        ws_consumer16<Cfg, WN, NCONS, false, true>(a, lds0, lane, wave, id_first, id_end, S);
+    else
+        ws_consumer<Cfg, V, WN, NCONS, false, true>(a, lds0, lane, wave, id_first, id_end, S);
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+static hipError_t launch_chwb(const SpmmLaunchArgs& a, hipStream_t stream)
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    SpmmLaunchArgs b = a;
+    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    const int T = a.X * b.n_tiles;
+    int grid = a.num_cus > 0 ? a.num_cus : 256;
+    grid = (grid / 8) * 8;
+    const int need = ((T + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL((spconv_chwb_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid), dim3(Cfg::THREADS), Cfg::LDS_BYTES,
+                       stream, b);
+    return hipGetLastError();
+}
+
+template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
+static hipError_t prepare_chwb()
+{
+    using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
+    return hipFuncSetAttribute((const void*)spconv_chwb_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+}
+
+#define SHFLBW_CHWB(V, WN, NC, NP, KT, NS)                                                                             \
+    {                                                                                                                  \
+        V, WN* NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS>::LDS_BYTES, &launch_chwb<V, WN, NC, NP, KT, NS>,  \
+            &prepare_chwb<V, WN, NC, NP, KT, NS>                                                                       \
+    }
+
+static const ConvChwbKernel g_chwb[] = {
+    SHFLBW_CHWB(64, 128, 4, 4, 32, 4),
+    SHFLBW_CHWB(32, 128, 4, 4, 32, 4),
+    SHFLBW_CHWB(16, 128, 4, 4, 32, 4),
+    SHFLBW_CHWB(128, 64, 4, 4, 32, 6),
+};
+
+const ConvChwbKernel* conv_chwb_kernel(int V)
+{
+    for (const ConvChwbKernel& k : g_chwb)
+        if (k.V == V) return &k;
+    return nullptr;
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>

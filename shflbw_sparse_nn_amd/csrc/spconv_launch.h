@@ -74,10 +74,22 @@ struct ConvFusedKernel {
 };
 const ConvFusedKernel* conv_fused_kernel(int V);
 // cache lines of synchronisation words the fused form needs for a problem with `slabs` column tiles
-// floor(2^32 / d) for fast_divmod on the device
-inline unsigned udiv_magic(int d) { return d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / (unsigned)d); }
 constexpr int CONV_LINE_SLAB0 = 27; // first of the two lines per column tile
 inline int conv_sync_lines(int slabs) { return CONV_LINE_SLAB0 + 2 * slabs; }
+
+// Batch-innermost (C-H-W-B in, F-H-W-B out) form of the convolution: the copy into padded phase planes and the
+// role-split kernel whose epilogue writes compact output rows.
+hipError_t launch_chwb_to_planes(const half_t* in, half_t* planes, int B, int H, int W, int C, int R, int S, int stride,
+                                 int PHX, int PW, int pitch, hipStream_t stream);
+struct ConvChwbKernel {
+    int V;
+    int BN;
+    int threads;
+    int lds_bytes;
+    hipError_t (*launch)(const SpmmLaunchArgs&, hipStream_t);
+    hipError_t (*prepare)();
+};
+const ConvChwbKernel* conv_chwb_kernel(int V);
 
 // Stages 1 and 3 of the plane form of the convolution: NHWC input -> channel-major padded planes (one per
 // stride phase, `copies` = 1 or 2 with a copy moved by one value, rows of `pitch` values), and the

@@ -19,6 +19,9 @@ struct SpmmLaunchArgs {
     int ldb_bytes;          // bytes between rows of B one id apart (N * 2 for a dense row-major B)
     const half_t* C;
     half_t* D;
+    int ldd;                // values between two rows of C and D (N for the SpMM)
+    int dmap_row, dmap_valid; // batch-innermost convolution only: see output_column()
+    unsigned dmap_magic;      // udiv magic of dmap_row
     float alpha, beta;
     int num_cus; // compute units of the device (persistent kernels size their grid with it)
     int img_cols, img_skip; // convolution only: column m of the GEMM is plane position m + (m / img_cols) * img_skip

@@ -107,6 +107,18 @@ __device__ __forceinline__ void tile_done_signal(const SpmmLaunchArgs& a, int nt
     }
 }
 
+// Convolution over batch-innermost feature maps: the columns of the GEMM are the positions (i, j, b) of a padded
+// output grid, a.dmap_row of them per grid row, of which the first a.dmap_valid are output values.  Maps a column
+// (a multiple of 8; dmap_row and dmap_valid are multiples of 8 too) to its column in the compact output row and
+// says whether it is one.
+__device__ __forceinline__ bool output_column(const SpmmLaunchArgs& a, int& col)
+{
+    int q, r;
+    fast_divmod(col, a.dmap_row, a.dmap_magic, q, r);
+    col = q * a.dmap_valid + r;
+    return r < a.dmap_valid;
+}
+
 // Walks the tile ids id, id+S, ... < end of one workgroup and keeps the descriptor of the
 // current and of the following tile in scalar registers, so a tile switch never waits for memory.
 struct TileWalker {
@@ -145,7 +157,7 @@ struct TileWalker {
 // per-wave epilogue area; the barrier protocol is: after START_BARRIERS start-up barriers, barrier
 // number t (counted from 0) is passed once stage t of the workgroup's stage stream is complete in
 // LDS; a consumer executes one barrier before its first stage and one more per stage.
-template <typename Cfg, int V, int WN, int NCONS, bool SIGNAL = false>
+template <typename Cfg, int V, int WN, int NCONS, bool SIGNAL = false, bool DMAP = false>
 __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
                                             int id_end, int S)
 {
@@ -293,7 +305,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
 #pragma unroll
                 for (int it = 0; it < NIT; it++) {
                     const int rr = mb * 32 + hh * ER + it * RPS + lane / PR;
-                    roff[it] = (size_t)__shfl(rid[rr >> 6], rr & 63) * N;
+                    roff[it] = (size_t)__shfl(rid[rr >> 6], rr & 63) * a.ldd;
                 }
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
@@ -313,8 +325,10 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
 #pragma unroll
                     for (int it = 0; it < NIT; it++)
                         v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * RPS * Cfg::EPI_ROWB);
-                    const int col = col0 + nb * 32;
-                    if (col < N) {
+                    int col = col0 + nb * 32;
+                    bool keep = col < N;
+                    if (DMAP) keep = keep && output_column(a, col);
+                    if (keep) {
                         if (ADDC) {
 #pragma unroll
                             for (int it = 0; it < NIT; it++) c[it] = *(const half8_t*)(a.C + roff[it] + col);
@@ -355,7 +369,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
 // Consumer role for block height 16: 16x16x32 tiles, one 32-slot step per LDS stage, same barrier
 // protocol and ring as ws_consumer.  Wave `cw` owns the 16 x WN sub-tile at column cw*WN.  A lane of
 // the result holds output row lane % 16 and, per 16-column block, the 4 columns 4*(lane/16) + 0..3.
-template <typename Cfg, int WN, int NCONS, bool SIGNAL = false>
+template <typename Cfg, int WN, int NCONS, bool SIGNAL = false, bool DMAP = false>
 __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
                                               int id_end, int S)
 {
@@ -441,7 +455,7 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
         const uint32_t rd = epi + (lane >> 3) * EROWB + (lane & 7) * 16;
         size_t roff[2];
 #pragma unroll
-        for (int it = 0; it < 2; it++) roff[it] = (size_t)__shfl(orow, it * 8 + (lane >> 3)) * N;
+        for (int it = 0; it < 2; it++) roff[it] = (size_t)__shfl(orow, it * 8 + (lane >> 3)) * a.ldd;
 #pragma unroll
         for (int h = 0; h < WN / 64; h++) {
 #pragma unroll
@@ -454,8 +468,10 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
             half8_t v[2];
 #pragma unroll
             for (int it = 0; it < 2; it++) v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * 8 * EROWB);
-            const int col = n0 + cw * WN + h * 64 + (lane & 7) * 8;
-            if (col < N) {
+            int col = n0 + cw * WN + h * 64 + (lane & 7) * 8;
+            bool keep = col < N;
+            if (DMAP) keep = keep && output_column(a, col);
+            if (keep) {
                 if (beta != 0.f) {
                     half8_t c[2];
 #pragma unroll

@@ -173,6 +173,14 @@ class BlockwiseSpFilter(BlockwiseSpMatrix):
         capi.check(self._lib.shflbw_spconv_host_reference(self._h, Bn, H, W, stride, x.ctypes.data, out.ctypes.data))
         return out
 
+    def host_reference_chwb(self, x_chwb, stride):
+        """The same over the reference's tensors: input [C][H][W][B], output fp32 [F][H][W][B], H and W bounding both."""
+        x = np.ascontiguousarray(x_chwb, dtype=np.float16)
+        _, H, W, Bn = x.shape
+        out = np.empty((self.info.F, H, W, Bn), dtype=np.float32)
+        capi.check(self._lib.shflbw_spconv_host_reference_chwb(self._h, Bn, H, W, stride, x.ctypes.data, out.ctypes.data))
+        return out
+
 
 class SpmmBlockwiseOp:
     """initialize(spmat, N, B, [C,] D) then op() launches on `stream` (asynchronous)."""
@@ -204,9 +212,14 @@ class SpconvBlockwiseOp:
         self._state = capi.SpconvState()
         self._variant = variant
 
-    def initialize(self, spfilter, B, H, W, stride, IFMap, OFMap):
-        capi.check(self._lib.shflbw_spconv_init_variant(C.byref(self._state), spfilter._h, B, H, W, stride, IFMap,
-                                                        OFMap, self._variant))
+    def initialize(self, spfilter, B, H, W, stride, IFMap, OFMap, batch_innermost=False):
+        """batch_innermost=True: the reference's C-H-W-B / F-H-W-B tensors and its bounds rule (H, W bound input and
+        output alike); the form is then fixed."""
+        if batch_innermost:
+            capi.check(self._lib.shflbw_spconv_init_chwb(C.byref(self._state), spfilter._h, B, H, W, stride, IFMap, OFMap))
+        else:
+            capi.check(self._lib.shflbw_spconv_init_variant(C.byref(self._state), spfilter._h, B, H, W, stride, IFMap,
+                                                            OFMap, self._variant))
         self._keep = spfilter
         return self._state
 

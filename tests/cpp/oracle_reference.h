@@ -17,6 +17,9 @@ int oracle_spmm_reference(int nrow, int ncol, int brow, int bcol, const int* ind
 int oracle_spconv_reference_nhwc(int F, int R, int S, int C, int brow, const int* indptr, const int* indices,
                                  const uint16_t* values, const int* row_permute_ids, int B, int H, int W, int stride,
                                  int pad_h, int pad_w, const uint16_t* IFMap, float* OFMap_ref, int nthreads);
+int oracle_spconv_reference_chwb(int F, int R, int S, int C, int brow, int bcol, const int* indptr, const int* indices,
+                                 const uint16_t* values, const int* row_permute_ids, int B, int H, int W, int stride,
+                                 const uint16_t* IFMap, float* OFMap_ref);
 }
 
 template <typename T>
@@ -49,6 +52,22 @@ void oracle_reference(BlockwiseSpFilter<T>& f, int B, int H, int W, int stride, 
                                           f.S / 2, reinterpret_cast<const uint16_t*>(IFMap.data()), OFMap_ref.data(), 0);
     if (rc != 0) {
         std::cerr << "oracle_spconv_reference_nhwc failed: " << rc << std::endl;
+        std::exit(EXIT_FAILURE);
+    }
+}
+
+// the reference's own tensors: C-H-W-B in, F-H-W-B out, H and W bounding both (spconv/blockwise_format.h:111-128)
+template <typename T>
+void oracle_reference_batch_first(BlockwiseSpFilter<T>& f, int B, int H, int W, int stride, const std::vector<T>& IFMap,
+                                  std::vector<float>& OFMap_ref)
+{
+    OFMap_ref.assign(static_cast<size_t>(B) * H * W * f.F, 0.f);
+    int rc = oracle_spconv_reference_chwb(f.F, f.R, f.S, f.C, f.brow, f.bcol, f.indptr.data(), f.indices.data(),
+                                          reinterpret_cast<const uint16_t*>(f.values.data()),
+                                          f.row_permute ? f.row_permute_ids.data() : nullptr, B, H, W, stride,
+                                          reinterpret_cast<const uint16_t*>(IFMap.data()), OFMap_ref.data());
+    if (rc != 0) {
+        std::cerr << "oracle_spconv_reference_chwb failed: " << rc << std::endl;
         std::exit(EXIT_FAILURE);
     }
 }

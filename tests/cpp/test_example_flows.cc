@@ -2,7 +2,7 @@
 // linked against libblock_sparse.a only (no test oracle): header-form SpMM with D = A*B + C and the
 // library's own get_host_reference as the check (example/spmm.blockwise.cu:17-52), a weight loaded from
 // its text dump (example/load_bsr.spmm.blockwise.cu:10-28), and the header-form convolution
-// (example/spconv.blockwise.cu:17-52; feature maps are NHWC here, so the comparison walks NHWC).
+// (example/spconv.blockwise.cu:17-52, once over NHWC feature maps and once over the reference's own C-H-W-B / F-H-W-B).
 // A fourth flow checks that dump() of a synced weight is read-only: sync, initialize, dump, launch.
 #include <cmath>
 #include <sstream>
@@ -93,6 +93,48 @@ static bool spconv_flow(int stride, bool filter_permute)
     return ok;
 }
 
+// example/spconv.blockwise.cu as it stands: C-H-W-B input allocated for (H*stride) x (W*stride), F-H-W-B output, the
+// comparison indexed nn + (ww + (hh + ff*H)*W)*B
+static bool spconv_flow_reference_layout(int stride)
+{
+    const int B = 32, H = 14, W = 14, C = 256, F = 256, R = 3, S = 3, block_sz = 32;
+    BlockwiseSpFilter<half> spfilter;
+    spfilter.init_random(F, R, S, C, block_sz, 1, 0.2f, false, 2021u);
+    spfilter.fmap_layout = fmap_batch_first;
+    spfilter.transform_and_sync_device();
+
+    CudaRandomArray<half> IFMap;
+    CudaZerosArray<half> OFMap;
+    IFMap.initialize(B * (H * stride) * (W * stride) * C);
+    OFMap.initialize(B * H * W * F);
+    IFMap.sync_device();
+    OFMap.sync_device();
+
+    SpconvBlockwiseOp<ShapeBase<block_sz, 128, 32>, ShapeBase<32, 32, 32>, ShapeBase<16, 16, 16>, 3> op;
+    op.initialize(spfilter, B, H, W, stride, IFMap.device_ptr, OFMap.device_ptr);
+    op();
+    HIP_CHECK(hipDeviceSynchronize());
+    OFMap.sync_host();
+
+    std::vector<float> OFMap_ref(B * H * W * F);
+    get_host_reference<half>(spfilter, B, H, W, stride, IFMap.host_array, OFMap_ref, filter_channel_first);
+    bool passed = true;
+    for (int nn = 0; nn < B; nn++)
+        for (int hh = 0; hh < H; hh++)
+            for (int ww = 0; ww < W; ww++)
+                for (int ff = 0; ff < F; ff++) {
+                    const int idx = nn + (ww + (hh + ff * H) * W) * B;
+                    const float o = static_cast<float>(OFMap.host_array[idx]), o_ref = OFMap_ref[idx];
+                    if (!(std::fabs(o_ref - o) <= 1e-3f * std::fabs(o_ref))) {
+                        if (passed) printf("n = %d, h = %d, w = %d, f = %d, result %f != %f\n", nn, hh, ww, ff, o, o_ref);
+                        passed = false;
+                    }
+                }
+    std::cout << "spconv example, reference layout, stride " << stride << " (" << spfilter.config_str << ")"
+              << (passed ? " Passed" : " Failed") << "\n";
+    return passed;
+}
+
 int main()
 {
     int failures = 0;
@@ -119,6 +161,8 @@ int main()
     }
     failures += !spconv_flow(1, false);
     failures += !spconv_flow(2, true);
+    failures += !spconv_flow_reference_layout(1);
+    failures += !spconv_flow_reference_layout(2);
     std::cout << (failures ? "FAILED " : "ALL PASSED ") << failures << " failure(s)\n";
     return failures ? EXIT_FAILURE : EXIT_SUCCESS;
 }

@@ -3,6 +3,7 @@
 // density 0.1, seed 2021), with NHWC feature maps and a true stride: the input is
 // (h*stride) x (w*stride), the output h x w.  Plain and filter-permuted weights.  The batch is
 // cut to 16 images to keep the CPU oracle quick; N = 16*14*14 = 3136 still leaves a ragged tile.
+// Then the same filters over the reference's own batch-innermost tensors.
 #include <cmath>
 #include <tuple>
 #include "block_sparse/cuda_array.h"
@@ -75,6 +76,22 @@ static int test_block_size(int block_sz, int n, int h, int w, int c, int f, int 
         bool ok1 = verify(*e.init, *e.exec, permuted, n, h_in, w_in, stride, IFMap, OFMap, ref_permuted);
         std::cout << e.name << " " << plain.config_str << " n=" << n << " h=" << h << " w=" << w << " stride=" << stride
                   << (ok0 ? " Passed" : " Failed") << " | permuted" << (ok1 ? " Passed" : " Failed") << "\n";
+        failures += !ok0 + !ok1;
+    }
+
+    // the same filters over the reference's own tensors (C-H-W-B in, F-H-W-B out, h x w bounding both)
+    plain.fmap_layout = permuted.fmap_layout = fmap_batch_first;
+    CudaRandomArray<half> IFMap_bf;
+    IFMap_bf.initialize(n * h * w * c);
+    oracle_reference_batch_first<half>(plain, n, h, w, stride, IFMap_bf.host_array, ref_plain);
+    oracle_reference_batch_first<half>(permuted, n, h, w, stride, IFMap_bf.host_array, ref_permuted);
+    for (const TableEntry& e : table) {
+        if (e.block_sz != block_sz) continue;
+        bool ok0 = verify(*e.init, *e.exec, plain, n, h, w, stride, IFMap_bf, OFMap, ref_plain);
+        bool ok1 = verify(*e.init, *e.exec, permuted, n, h, w, stride, IFMap_bf, OFMap, ref_permuted);
+        std::cout << e.name << " batch-first " << plain.config_str << " n=" << n << " h=" << h << " w=" << w
+                  << " stride=" << stride << (ok0 ? " Passed" : " Failed") << " | permuted" << (ok1 ? " Passed" : " Failed")
+                  << "\n";
         failures += !ok0 + !ok1;
     }
     return failures;

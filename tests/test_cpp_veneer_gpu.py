@@ -38,7 +38,7 @@ def test_reference_example_flows(torch_gpu):
     # the reference's three example programs as flows over this library's headers, checked with the library's
     # own get_host_reference, linked against libblock_sparse.a only
     out = _run("test_example_flows", 100)
-    assert out.count("Passed") == 5 and "Failed" not in out
+    assert out.count("Passed") == 7 and "Failed" not in out
 
 
 BENCH = os.path.join(ROOT, "shflbw_sparse_nn_amd", "block_sparse", "benchmark")

@@ -213,3 +213,16 @@ def test_library_spconv_host_reference_equals_the_oracle(stride, R, Sx):
     f = S.BlockwiseSpFilter()
     f.set(F, R * Sx * Cc, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"], R, Sx, Cc)
     np.testing.assert_array_equal(f.host_reference(x, stride), P.conv_oracle(w, R, Sx, Cc, x, stride))
+
+
+@pytest.mark.parametrize("stride,R,Sx,permute", [(1, 3, 3, True), (2, 3, 3, True), (1, 5, 1, False)])
+def test_library_reference_layout_host_reference_equals_the_oracle(stride, R, Sx, permute):
+    import workloads as P
+    Cc, F, V, Bn, H, W = 12, 64, 32, 8, 7, 6
+    w = P.make_weight(F, R * Sx * Cc, V, 0.3, permute, 11, dist=("normal", 1.0))
+    x = np.random.default_rng(4).standard_normal((Cc, H, W, Bn)).astype(np.float16)
+    f = S.BlockwiseSpFilter()
+    f.set(F, R * Sx * Cc, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"], R, Sx, Cc)
+    ref = O.spconv_reference_chwb(F, R, Sx, Cc, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"],
+                                  Bn, H, W, stride, x)
+    np.testing.assert_array_equal(f.host_reference_chwb(x, stride), ref)

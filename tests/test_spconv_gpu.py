@@ -136,3 +136,44 @@ def test_non_finite_input_does_not_leak_through_padding(torch_gpu):
         assert np.array_equal(np.isnan(got), np.isnan(ref)), "form %d: NaN pattern differs" % variant
         ok = ~np.isnan(ref)
         np.testing.assert_array_equal(got[ok], ref[ok], err_msg="form %d" % variant)
+
+
+@pytest.mark.parametrize("Bn,H,W,C,F,R,S,stride,V,d,permute", [
+    (16, 14, 14, 64, 128, 3, 3, 1, 64, 0.2, True),
+    (16, 14, 14, 64, 128, 3, 3, 2, 64, 0.2, True),    # the reference's "strided" case: taps beyond H x W read zero
+    (8, 7, 9, 20, 64, 3, 3, 1, 32, 0.3, False),       # ragged extents, C not a multiple of 8
+    (8, 6, 10, 16, 32, 5, 3, 2, 16, 0.4, True),       # block height 16, 5 x 3 filter
+    (24, 5, 5, 8, 128, 1, 1, 1, 128, 0.5, True),      # 1 x 1 filter: no padding columns at all
+    (8, 12, 12, 16, 64, 3, 3, 3, 32, 0.3, True),      # stride 3
+])
+def test_reference_layout_exact(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute):
+    """The operator over the reference's own tensors (C-H-W-B in, F-H-W-B out, H and W bounding both) against the
+    oracle's literal restatement of spconv/blockwise_format.h:55-132, bit for bit on integer data."""
+    import shflbw_sparse_nn_amd as Sx
+    torch = torch_gpu
+    w = P.make_weight(F, R * S * C, V, d, permute, 2021, integer=True)
+    x = np.random.default_rng(9).integers(-4, 5, size=(C, H, W, Bn)).astype(np.float16)
+    ref = O.float_to_half(O.spconv_reference_chwb(F, R, S, C, V, 1, w["indptr"], w["indices"], w["values"],
+                                                  w["row_permute_ids"], Bn, H, W, stride, x))
+    f = P.upload_weight(w, R, S, C, cls=Sx.BlockwiseSpFilter)
+    dX = P.to_dev(torch, x)
+    dY = torch.full((F, H, W, Bn), float("nan"), dtype=torch.float16, device="cuda")
+    op = Sx.SpconvBlockwiseOp()
+    op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr(), batch_innermost=True)
+    for _ in range(2):  # a second launch over the same scratch
+        op(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    got = dY.cpu().numpy()
+    assert not np.isnan(got.astype(np.float32)).any(), "output elements left unwritten"
+    np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+def test_reference_layout_needs_a_batch_of_eights(torch_gpu):
+    import shflbw_sparse_nn_amd as Sx
+    from shflbw_sparse_nn_amd import capi
+    w = P.make_weight(64, 9 * 8, 32, 0.3, True, 3, integer=True)
+    f = P.upload_weight(w, 3, 3, 8, cls=Sx.BlockwiseSpFilter)
+    t = torch_gpu.zeros(4096, dtype=torch_gpu.float16, device="cuda")
+    with pytest.raises(capi.ShflbwError) as e:
+        Sx.SpconvBlockwiseOp().initialize(f, 4, 5, 5, 1, t.data_ptr(), t.data_ptr(), batch_innermost=True)
+    assert e.value.status == capi.ERR_SHAPE
