@@ -168,6 +168,7 @@ typedef struct shflbw_spmm_state {
     int brow;
     int ldb_bytes; /* distance in bytes between two rows of B that are one kept-column id apart: N * 2 */
     const void* zero_row; /* 1 KiB of zeros inside the library (device memory): gathered for the padding slots */
+    const int* packed_slab; /* the ids as LDS offsets for the tile variants that hold B in LDS; NULL when the weight has too many columns */
 } shflbw_spmm_state;
 
 /* C may be NULL when beta == 0.  variant < 0 selects automatically. */

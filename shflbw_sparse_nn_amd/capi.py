@@ -56,7 +56,8 @@ class SpmmState(C.Structure):
     _fields_ = [("shared_mem_size", C.c_size_t), ("grid_dim", C.c_uint * 3), ("block_dim", C.c_uint * 3),
                 ("init_success", C.c_int), ("variant", C.c_int), ("args", _SpmmArgs),
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("packed_indices_pm", C.c_void_p),
-                ("panel_ptr", C.c_void_p), ("brow", C.c_int), ("ldb_bytes", C.c_int), ("zero_row", C.c_void_p)]
+                ("panel_ptr", C.c_void_p), ("brow", C.c_int), ("ldb_bytes", C.c_int), ("zero_row", C.c_void_p),
+                ("packed_slab", C.c_void_p)]
 
 
 class _SpconvArgs(C.Structure):

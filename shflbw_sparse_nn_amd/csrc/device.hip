@@ -30,7 +30,7 @@ namespace shflbw {
 void clear_device(shflbw_weight* w)
 {
     void** bufs[] = {&w->d_meta, &w->d_values, &w->d_group_ptr, &w->d_packed_indices, &w->d_packed_indices_pm,
-                     &w->d_packed_values};
+                     &w->d_packed_values, &w->d_packed_slab};
     for (void** b : bufs) {
         if (*b) (void)hipFree(*b);
         *b = nullptr;
@@ -57,7 +57,8 @@ int upload(shflbw_weight* w)
         (rc = upload_one(&w->d_packed_indices, w->packed_indices.data(), w->packed_indices.size() * sizeof(int))) ||
         (rc = upload_one(&w->d_packed_indices_pm, w->packed_indices_pm.data(),
                          w->packed_indices_pm.size() * sizeof(int))) ||
-        (rc = upload_one(&w->d_packed_values, w->packed_values.data(), w->packed_values.size() * sizeof(uint16_t)))) {
+        (rc = upload_one(&w->d_packed_values, w->packed_values.data(), w->packed_values.size() * sizeof(uint16_t))) ||
+        (rc = upload_one(&w->d_packed_slab, w->packed_slab.data(), w->packed_slab.size() * sizeof(int)))) {
         clear_device(w);
         return rc;
     }
@@ -116,14 +117,38 @@ static bool spmm_variant_offsets32(const SpmmVariant* v) { return v && v->name[0
 // wide) variant of every block size first.  When its tiles would occupy at most half of the compute units,
 // the role-split variant with 256-column tiles is taken instead (twice the tiles; measured 15-25 % faster
 // there, 5-20 % slower once the wide tiles fill the chip).
-static int auto_spmm_variant(int brow, int X, int N)
+// Block height 32 and at most SLAB_MAX_K columns: the slab variant moves less data between the L2 and the
+// compute units once a workgroup runs enough kept vectors over the 128 KiB slab it has to load first.  Taken
+// when a workgroup's panels keep at least 6 vectors per column of A on average (below that the slab load
+// dominates: measured 7-30 % slower at 1.6) and A has at least 512 columns (with fewer, B fits the L2 and
+// the gathers of the role-split kernel all hit) and the packed A is at most 5 MB (all workgroups of an XCD
+// stream all of A from its 4 MB L2; at 6.7 MB the variant was 25 % slower).  Measured 2-28 % faster inside
+// these bounds (M = 4096, K = 1024, N = 4096, density 0.2: 15.1 against 16.5 us).
+static int auto_spmm_variant(const shflbw_weight* w, int N)
 {
+    const int brow = w->brow, X = w->nrow / w->brow;
+    int count = 0;
+    const SpmmVariant* all = spmm_variants(&count);
+    if (brow == 32 && !w->packed_slab.empty() && w->ncol >= 512 && X > 0) {
+        int seen = 0;
+        for (int i = 0; i < count; i++) {
+            if (all[i].V != brow) continue;
+            if (all[i].max_k >= w->ncol) {
+                const int cus = (device_compute_units() / 8) * 8;
+                const int n_tiles = (N + all[i].BN - 1) / all[i].BN;
+                const int chunks = std::max(1, std::min(X, cus / n_tiles)); // as the launcher deals the panels
+                const double panels_per_wg = (double)X / chunks;
+                const double vectors_per_column = panels_per_wg * w->nnzb / ((double)X * w->ncol);
+                if (vectors_per_column >= 6.0 && (double)w->nnzb * brow * 2 <= 5.0e6) return seen;
+            }
+            seen++;
+        }
+    }
     const SpmmVariant* first = find_spmm_variant(brow, 0, nullptr);
     if (!first || first->BN != 512) return 0;
     const long wide_tiles = (long)X * ((N + 511) / 512);
     if (wide_tiles > device_compute_units() / 2) return 0;
-    int count = 0, seen = 0;
-    const SpmmVariant* all = spmm_variants(&count);
+    int seen = 0;
     for (int i = 0; i < count; i++) {
         if (all[i].V != brow) continue;
         const bool role_split = all[i].name[0] == 'w'; // "ws..." names
@@ -189,6 +214,8 @@ static void fill_spmm_launch_args(const shflbw_spmm_state* state, int BN, SpmmLa
     a.packedA = (const half8_t*)state->packed_values;
     a.kidx = state->packed_indices;
     a.kidx_pm = state->packed_indices_pm;
+    a.slab_ids = state->packed_slab;
+    a.slab_chunks = 1;
     a.panel_desc = state->panel_ptr;
     a.row_ids = state->args.A_row_indices;
     a.B = (const half_t*)state->args.B;
@@ -261,7 +288,7 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     // the role-split kernels address the rows of B with 32-bit byte offsets
     const bool wide_b = (unsigned long long)w->ncol * (unsigned long long)N * 2ull + (unsigned long long)N * 2ull > 0xffffffffull;
     if (variant < 0) {
-        variant = auto_spmm_variant(w->brow, X, N);
+        variant = auto_spmm_variant(w, N);
         if (wide_b) { // first variant of this block size with 64-bit addressing
             int n = 0;
             find_spmm_variant(w->brow, 0, &n);
@@ -275,6 +302,11 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     const SpmmVariant* v = find_spmm_variant(w->brow, variant, nullptr);
     if (!v) {
         set_error("spmm_init: no tile variant %d for block size %d", variant, w->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (v->max_k > 0 && (w->ncol > v->max_k || w->packed_slab.empty())) {
+        set_error("spmm_init: tile variant %s holds all rows of B in LDS: at most %d columns of A (got %d)", v->name,
+                  v->max_k, w->ncol);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     if (wide_b && spmm_variant_offsets32(v)) {
@@ -300,6 +332,7 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     state->packed_values = w->d_packed_values;
     state->packed_indices = (const int*)w->d_packed_indices;
     state->packed_indices_pm = (const int*)w->d_packed_indices_pm;
+    state->packed_slab = w->packed_slab.empty() ? nullptr : (const int*)w->d_packed_slab;
     state->panel_ptr = (const int*)w->d_group_ptr;
     state->brow = w->brow;
     state->ldb_bytes = N * 2;

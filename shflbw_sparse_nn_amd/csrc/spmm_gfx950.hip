@@ -21,6 +21,8 @@
 
 #include "kernel_common.h"
 #include "spmm_launch.h"
+#include <algorithm>
+#include "spmm_slab.h"
 #include "spmm_ws.h"
 
 namespace shflbw {
@@ -326,6 +328,38 @@ static hipError_t prepare_ws()
     }
 
 // ---------------------------------------------------------------------------------------
+// slab form (all rows of a 64-column slab of B in LDS): launcher
+// ---------------------------------------------------------------------------------------
+static hipError_t launch_slab(const SpmmLaunchArgs& a, hipStream_t stream)
+{
+    using Cfg = SpmmSlabCfg;
+    if (a.K > Cfg::MAX_K || !a.slab_ids || a.K <= 0) return hipErrorInvalidValue;
+    SpmmLaunchArgs b = a;
+    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    // the panels under one column tile are dealt to as many workgroups as it takes to give every compute unit a job
+    // ... and so that the panels of one wave have at most RID_REGS * 64 rows
+    const int cus = ((a.num_cus > 0 ? a.num_cus : 256) / 8) * 8;
+    const int rows_per_wg = Cfg::NW * Cfg::RID_REGS * 64;
+    b.slab_chunks = std::max(1, std::min(a.X, std::max(cus / b.n_tiles, (a.M + rows_per_wg - 1) / rows_per_wg)));
+    const int T = b.n_tiles * b.slab_chunks;
+    const int grid = std::min(cus, ((T + 7) / 8) * 8);
+    hipLaunchKernelGGL(spmm_shflbw_slab_kernel, dim3(grid), dim3(Cfg::THREADS), Cfg::lds_bytes(a.K), stream, b);
+    return hipGetLastError();
+}
+
+static hipError_t prepare_slab()
+{
+    return hipFuncSetAttribute((const void*)spmm_shflbw_slab_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               SpmmSlabCfg::LDS_MAX);
+}
+
+#define SHFLBW_SLAB_VARIANT()                                                                                     \
+    {                                                                                                             \
+        SpmmSlabCfg::V, SpmmSlabCfg::BN, SpmmSlabCfg::THREADS, SpmmSlabCfg::LDS_MAX, "slab32x64", &launch_slab,    \
+            &prepare_slab, SpmmSlabCfg::MAX_K                                                                     \
+    }
+
+// ---------------------------------------------------------------------------------------
 // variant table
 // ---------------------------------------------------------------------------------------
 template <int V, int WN, int NWAVES, int KT, int NSTAGE>
@@ -380,6 +414,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(32, 128, 2, 32, 3),
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
     SHFLBW_VARIANT(32, 64, 2, 32, 3),
+    SHFLBW_SLAB_VARIANT(), // weights of at most SLAB_MAX_K columns
     // block 16
     SHFLBW_WS_VARIANT(16, 128, 4, 4, 32, 4),
     // block 128

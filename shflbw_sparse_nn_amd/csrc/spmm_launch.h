@@ -12,6 +12,8 @@ struct SpmmLaunchArgs {
     const half8_t* packedA; // private image: A fragments in register order
     const int* kidx;        // private image: kept column ids, 64-slot padded per panel
     const int* kidx_pm;     // same ids, each 64-slot group reordered producer-major: [16p + 4j + r] = [16j + 4p + r]
+    const int* slab_ids;    // slab kernel only: the ids as LDS offsets of slab rows, [group][pair of slots][step][2]
+    int slab_chunks;        // slab kernel only: the panels are dealt to this many workgroups per column tile (launcher)
     const int* panel_desc;  // private image: per panel {MFMA k16 steps = ceil(nnz/16), first 64-slot group}
     const int* row_ids;     // M, or null when rows are not permuted
     const half_t* B;
@@ -38,6 +40,7 @@ struct SpmmVariant {
     const char* name;
     hipError_t (*launch)(const SpmmLaunchArgs&, hipStream_t);
     hipError_t (*prepare)(); // raises the dynamic-LDS limit of the kernel
+    int max_k;               // 0, or the most columns of A the variant takes (it holds all rows of B in LDS)
 };
 
 const SpmmVariant* spmm_variants(int* count);

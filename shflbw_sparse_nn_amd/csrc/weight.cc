@@ -152,6 +152,7 @@ static void mark_initialized(shflbw_weight* w)
     w->packed_indices.clear();
     w->packed_indices_pm.clear();
     w->packed_values.clear();
+    w->packed_slab.clear();
 }
 
 static int check_pattern(int nrow, int ncol, int brow, int bcol, int nnzb, const int* indptr, const int* indices,
@@ -229,15 +230,45 @@ int build_packed_image(shflbw_weight* w)
     w->packed_indices.assign(slots, 0);
     w->packed_indices_pm.assign(slots, 0);
     w->packed_values.assign(slots * V, 0);
+    const bool slab = V == 32 && w->ncol <= SLAB_MAX_K;
+    w->packed_slab.assign(slab ? slots : 0, 0);
     for (int i = 0; i < X; i++) {
         const int begin = w->indptr[i], nnz = w->indptr[i + 1] - begin;
         const size_t slot0 = (size_t)w->group_ptr[i] * 64;
         const int padded = (w->group_ptr[i + 1] - w->group_ptr[i]) * 64;
+        // Order of the panel's kept vectors in the image: ascending ids, except for the slab form.  There the four
+        // slab rows of slots 4j .. 4j+3 are read by one LDS instruction and should lie in four different bank
+        // groups (slab_bank_class): every quad takes the next id of each of the classes with the most ids left.
+        std::vector<int> ord(nnz);
+        for (int q = 0; q < nnz; q++) ord[q] = q;
+        if (slab) {
+            std::vector<int> of_class[4];
+            for (int q = nnz - 1; q >= 0; q--) of_class[slab_bank_class(w->indices[begin + q])].push_back(q); // back() = smallest id
+            for (int q = 0; q < nnz;) {
+                int cls[4] = {0, 1, 2, 3};
+                std::stable_sort(cls, cls + 4, [&](int x, int y) { return of_class[x].size() > of_class[y].size(); });
+                const int quad_end = std::min(nnz, q + 4);
+                for (int t = 0; q < quad_end; t++) {
+                    std::vector<int>& from = of_class[cls[t % 4]];
+                    if (from.empty()) continue; // fewer than four classes left: the fullest ones give a second id
+                    ord[q++] = from.back();
+                    from.pop_back();
+                }
+            }
+        }
         for (int q = 0; q < padded; q++)
-            w->packed_indices[slot0 + q] = q < nnz ? w->indices[begin + q] : -1; // padding: gathered from a row of zeros
+            w->packed_indices[slot0 + q] = q < nnz ? w->indices[begin + ord[q]] : -1; // padding: gathered from a row of zeros
         for (int q = 0; q < padded; q++) {
             const int grp = q / 64, j = (q % 64) / 16, p = (q % 16) / 4, r = q % 4;
             w->packed_indices_pm[slot0 + grp * 64 + 16 * p + 4 * j + r] = w->packed_indices[slot0 + q];
+        }
+        // slab form: a lane of the consumer addresses slots s and s + 4 of every 16-slot step, s = 8 (pair / 4) +
+        // pair % 4 for its pair number 0..7; the eight offsets a lane needs for the four steps of a group are
+        // stored together, [group][pair][step][s, s + 4]
+        for (int q = 0; slab && q < padded; q++) {
+            const int grp = q / 64, step = (q % 64) / 16, s = q % 16;
+            const int pair = (s / 8) * 4 + s % 4, hi = (s % 8) / 4;
+            w->packed_slab[slot0 + grp * 64 + pair * 8 + step * 2 + hi] = slab_row_offset(w->packed_indices[slot0 + q], w->ncol);
         }
         uint16_t* dst = w->packed_values.data() + slot0 * V;
         const uint16_t* src = w->values.data() + (size_t)begin * V;
@@ -247,7 +278,7 @@ int build_packed_image(shflbw_weight* w)
                 const int s = q / 16, half_k = (q % 16) / 8, j = q % 8;
                 for (int r = 0; r < V; r++) {
                     const int mb = r / 32, lane = half_k * 32 + r % 32;
-                    dst[(((size_t)s * MB + mb) * 64 + lane) * 8 + j] = src[(size_t)q * V + r];
+                    dst[(((size_t)s * MB + mb) * 64 + lane) * 8 + j] = src[(size_t)ord[q] * V + r];
                 }
             }
         } else {
@@ -255,7 +286,7 @@ int build_packed_image(shflbw_weight* w)
                 const int s = q / 32, quarter = (q % 32) / 8, j = q % 8;
                 for (int r = 0; r < 16; r++) {
                     const int lane = quarter * 16 + r;
-                    dst[((size_t)s * 64 + lane) * 8 + j] = src[(size_t)q * 16 + r];
+                    dst[((size_t)s * 64 + lane) * 8 + j] = src[(size_t)ord[q] * 16 + r];
                 }
             }
         }

@@ -29,6 +29,9 @@ struct shflbw_weight {
     std::vector<int> packed_indices; // 64 * group_ptr[X]; tail slots hold -1 (a row of zeros)
     std::vector<int> packed_indices_pm; // each 64-slot group reordered: [16p + 4j + r] = packed_indices[16j + 4p + r]
     std::vector<uint16_t> packed_values; // 64 * brow * group_ptr[X]; MFMA fragment order, tail zero
+    // slab form of the SpMM (block sizes 32 and 64, ncol <= SLAB_MAX_K; empty otherwise): the ids of every 64-slot
+    // group as LDS byte offsets of slab rows, in the order the lanes of a wave load them (see build_packed_image)
+    std::vector<int> packed_slab;
 
     bool initialized = false, device_synced = false;
     std::string config_str;
@@ -40,6 +43,7 @@ struct shflbw_weight {
     void* d_packed_indices = nullptr;
     void* d_packed_indices_pm = nullptr;
     void* d_packed_values = nullptr;
+    void* d_packed_slab = nullptr;
 
     // Device scratch of the convolution (layout-transformed input, filter-major result, the kept-column ids
     // rewritten as plane offsets, synchronisation words): one allocation per distinct (form, geometry, input
@@ -67,6 +71,21 @@ uint16_t float_to_half(float f);
 
 // k-extent of one MFMA step for a block size: 32x32x16 tiles for V >= 32, 16x16x32 for V == 16
 inline int mfma_kstep(int brow) { return brow >= 32 ? 16 : 32; }
+
+// Geometry of the slab form of the SpMM: a workgroup holds up to SLAB_MAX_K rows of SLAB_ROW_BYTES bytes (64 columns)
+// of B in LDS, one more row of zeros behind them (rounded up to a multiple of 8 rows) for the padding slots.
+constexpr int SLAB_ROW_BYTES = 128;
+constexpr int SLAB_MAX_K = 1112;
+// LDS byte offset of what slot id `k` of a weight with `ncol` columns reads: the start of slab row k with the XOR key
+// of the row, (k / 2) % 4, in the position of the 32-byte unit; padding slots (k < 0) read the row of zeros.
+inline int slab_row_offset(int k, int ncol)
+{
+    return k < 0 ? ((ncol + 7) & ~7) * SLAB_ROW_BYTES : k * SLAB_ROW_BYTES + (((k >> 1) & 3) << 5);
+}
+
+// Which quarter of the LDS banks the 64 bytes of slab row k that one transposing read touches fall into (the other
+// 64 bytes of the row: the same quarter with the lowest bit flipped): rows of different class never collide.
+inline int slab_bank_class(int k) { return (k & 1) * 2 + ((k >> 2) & 1); }
 
 // builds group_ptr / packed_indices / packed_values from the host arrays
 int build_packed_image(shflbw_weight* w);

@@ -168,3 +168,56 @@ def test_non_finite_activations_do_not_leak_through_padding(torch_gpu, V):
         assert np.array_equal(np.isnan(got), np.isnan(ref)), "variant %d: NaN pattern differs" % variant
         ok = ~np.isnan(ref)
         np.testing.assert_array_equal(got[ok], ref[ok], err_msg="variant %d" % variant)
+
+
+def _slab_variant(V):
+    names = S.spmm_variants(V)
+    hits = [i for i, n in enumerate(names) if n.startswith("slab")]
+    assert len(hits) == 1, names
+    return hits[0]
+
+
+@pytest.mark.parametrize("M,N,K,V,d,permute", [
+    (4096, 4096, 1024, 32, 0.2, True),    # cfg2 shape: four workgroups per column tile, four panels per wave
+    (1024, 960, 1024, 32, 0.1, True),     # ragged N: the last column tile is half empty
+    (2048, 1024, 777, 32, 0.15, False),   # K not a multiple of 8: filler rows between the last row and the zeros
+    (64, 64, 8, 32, 1.0, True),           # one column tile, two panels, one step each
+    (256, 24000, 96, 32, 0.5, True),      # more column tiles than compute units: workgroups refill the slab
+    (8192, 128, 1112, 32, 0.05, True),    # the largest K the LDS takes; 256 panels over two column tiles
+    (4096, 512, 512, 32, 0.02, True),     # about ten kept vectors a panel: groups with one to three steps, empty panels
+    (96, 8, 40, 32, 0.6, True),           # N smaller than a piece of the second 32-column block
+])
+def test_slab_variant_exact(torch_gpu, M, N, K, V, d, permute):
+    """The variant that keeps all rows of a 64-column slab of B in LDS (weights of few columns), forced here on
+    shapes that exercise its job loop, its group stream across panels and its row of zeros."""
+    _exact_case(torch_gpu, M, N, K, V, d, permute, _slab_variant(V))
+
+
+def test_slab_variant_empty_panels_and_c(torch_gpu):
+    V = 32
+    M, N, K = 8 * V, 200, 128
+    X = M // V
+    counts = np.array([0, 0, 5, 0, 70, 1, 0, 0])  # leading, inner and trailing panels without a kept vector
+    indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rng = np.random.default_rng(5)
+    indices = np.concatenate([np.sort(rng.choice(K, c, replace=False)) for c in counts]).astype(np.int32)
+    w = dict(nrow=M, ncol=K, brow=V, bcol=1, nnzb=int(counts.sum()), indptr=indptr, indices=indices,
+             values=rng.integers(-4, 5, size=int(counts.sum()) * V).astype(np.float16),
+             row_permute_ids=O.row_permutation(M, 5))
+    assert X == len(counts)
+    B = P.make_dense(K, N, 3, integer=True)
+    Cm = P.make_dense(M, N, 3, integer=True, stream=3)
+    v = _slab_variant(V)
+    got = run_spmm(torch_gpu, w, B, variant=v)
+    np.testing.assert_array_equal(got.view(np.uint16), O.float_to_half(P.spmm_oracle(w, B)).view(np.uint16))
+    got = run_spmm(torch_gpu, w, B, Cmat=Cm, alpha=2.0, beta=-0.5, variant=v)
+    np.testing.assert_array_equal(got.view(np.uint16), O.float_to_half(P.spmm_oracle(w, B, Cm, 2.0, -0.5)).view(np.uint16))
+
+
+def test_slab_variant_refuses_wide_weights(torch_gpu):
+    from shflbw_sparse_nn_amd import capi
+    w = P.make_weight(64, 2048, 32, 0.1, True, 1, integer=True)
+    B = P.make_dense(2048, 64, 1, integer=True)
+    with pytest.raises(capi.ShflbwError) as e:
+        run_spmm(torch_gpu, w, B, variant=_slab_variant(32))
+    assert e.value.status == capi.ERR_UNSUPPORTED
