@@ -333,7 +333,9 @@ __global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __res
         [&](int o, int q, half8_t v) { // destination row = the pixel at position p0 + o, filters f0 + 8q ..
             const int n = p0 + o, f = f0 + q * 8;
             const int img = n / PS, rem = n % PS, ho = rem / PW, wo = rem % PW;
-            if (img < B && ho < Ho && wo < Wo && f < F) *(half8_t*)(out + ((size_t)(img * Ho + ho) * Wo + wo) * F + f) = v;
+            // streaming store: the output is not read again here and should not push the next launch's input out of the caches
+            if (img < B && ho < Ho && wo < Wo && f < F)
+                __builtin_nontemporal_store(v, (half8_t*)(out + ((size_t)(img * Ho + ho) * Wo + wo) * F + f));
         });
 }
 
