@@ -2,7 +2,7 @@
 """Benchmark of the Shfl-BW hot path on one MI355X.  Default workload: the headline SpMM, M = K = N = 4096,
 block size 64, density 0.1, row-permuted (BASELINE.json configs[1]).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg0|cfg1|cfg2|cfg3|cfg4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg0|cfg1|cfg2|cfg3|cfg4|refconv]
 
 A step is one `exec` of the operator on device-resident operands (fp16 in, fp32 accumulate, fp16 out):
 one launch for the SpMM configs (cfg0-cfg2), the whole convolution for cfg3/cfg4.  Timing follows the
@@ -115,7 +115,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500,
                     help="untimed launches before the timed ones; the shader clock needs about 10 ms of load to settle")
-    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D)")
+    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D) | refconv (the "
+                         "reference's own conv test case on its own tensor layout; not graded)")
     ap.add_argument("--variant", type=int, default=-1, help="force a kernel variant (default: library choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--traffic", default=None,
@@ -265,37 +266,45 @@ def bench_spmm(args, np, torch, S, P):
 
 
 def bench_conv(args, np, torch, S, P):
-    """The sparse Conv2D configs (cfg3, cfg4), NHWC; one step = one exec of the operator, i.e. every launch
-    the chosen form of the convolution puts on the stream.  Same JSON shape as the SpMM line."""
+    """The sparse Conv2D configs (cfg3, cfg4: NHWC; refconv: the reference's test case on its C-H-W-B / F-H-W-B
+    tensors); one step = one exec of the operator, i.e. every launch the chosen form of the convolution puts on
+    the stream.  Same JSON shape as the SpMM line."""
     from oracle import oracle as O  # correctness gate and CPU baseline only
     c = P.CONV_CONFIGS[args.config]
     B, H, W, C, F, R, Sx, stride, V, d = [c[k] for k in ("B", "H", "W", "C", "F", "R", "S", "stride", "V", "d")]
-    Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
+    batch_first = c.get("layout") == "chwb"
+    if batch_first:
+        Ho, Wo = H, W
+        in_shape, out_shape, variant = (C, H, W, B), (F, H, W, B), 4
+        oracle = lambda w, x, **kw: P.conv_oracle_batch_first(w, R, Sx, C, x, stride)
+    else:
+        Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
+        in_shape, out_shape, variant = (B, H, W, C), (B, Ho, Wo, F), max(args.variant, 0)
+        oracle = lambda w, x, **kw: P.conv_oracle(w, R, Sx, C, x, stride, **kw)
     npix = B * Ho * Wo
     stream = torch.cuda.current_stream()
-    variant = max(args.variant, 0)
 
     def make_op(w, x):
         f = P.upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
         dX = P.to_dev(torch, x)
-        dY = torch.full((B, Ho, Wo, F), float("nan"), dtype=torch.float16, device="cuda")
+        dY = torch.full(out_shape, float("nan"), dtype=torch.float16, device="cuda")
         op = S.SpconvBlockwiseOp(variant)
-        op.initialize(f, B, H, W, stride, dX.data_ptr(), dY.data_ptr())
+        op.initialize(f, B, H, W, stride, dX.data_ptr(), dY.data_ptr(), batch_innermost=batch_first)
         return op, f, dX, dY
 
     # correctness gate: bit-exact against the oracle on the integer twin
     wi = P.make_weight(F, R * Sx * C, V, d, True, 2021, integer=True)
-    xi = np.random.default_rng(2022).integers(-4, 5, size=(B, H, W, C)).astype(np.float16)
+    xi = np.random.default_rng(2022).integers(-4, 5, size=in_shape).astype(np.float16)
     opi, fi, dXi, dYi = make_op(wi, xi)
     opi(stream.cuda_stream)
     torch.cuda.synchronize()
-    ref_i = O.float_to_half(P.conv_oracle(wi, R, Sx, C, xi, stride))
+    ref_i = O.float_to_half(oracle(wi, xi))
     if not np.array_equal(dYi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
         print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
         sys.exit(1)
 
     w = P.make_weight(F, R * Sx * C, V, d, True, 2021, dist=c["w_dist"])
-    x = P.make_dense(B * H * W, C, 2021, dist=c["x_dist"]).reshape(B, H, W, C)
+    x = P.make_dense(B * H * W, C, 2021, dist=c["x_dist"]).reshape(in_shape)
     op, f, dX, dY = make_op(w, x)
     nnzb = w["nnzb"]
     eff_flops = 2.0 * nnzb * V * npix
@@ -313,10 +322,16 @@ def bench_conv(args, np, torch, S, P):
         XS = max(1, X // 8)
         sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
                    values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
-        cpu = cpu_baseline(lambda: P.conv_oracle(w, R, Sx, C, x, stride),
-                           lambda: P.conv_oracle(sub, R, Sx, C, x, stride, nthreads=1), eff_flops,
-                           2.0 * int(w["indptr"][XS]) * V * npix, "whole workload (%d panels)" % X,
-                           "the first %d panels" % XS, O.max_threads())
+        # the literal restatement of the reference's loop nest (batch-first layout) runs on one thread
+        if batch_first:  # one thread throughout: a bounded sample, the first panels, stands for the workload
+            cpu = cpu_baseline(lambda: oracle(sub, x), lambda: oracle(sub, x), 2.0 * int(w["indptr"][XS]) * V * npix,
+                               2.0 * int(w["indptr"][XS]) * V * npix, "the first %d of %d panels" % (XS, X),
+                               "the same", 1)
+        else:
+            cpu = cpu_baseline(lambda: oracle(w, x),
+                               lambda: oracle(sub, x, nthreads=1), eff_flops,
+                               2.0 * int(w["indptr"][XS]) * V * npix, "whole workload (%d panels)" % X,
+                               "the first %d panels" % XS, O.max_threads())
 
     eff_tflops = eff_flops / t / 1e12
     kernel = S.spconv_variant_name(variant)
@@ -328,8 +343,9 @@ def bench_conv(args, np, torch, S, P):
         "dtype": "f16 (fp32 accumulate)",
         "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter %s(%g), input %s(%g)"
                 % (c["w_dist"] + c["x_dist"]),
-        "config": {"workload": "%s: sparse Conv2D NHWC %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
-                               "nnzb=%d" % (args.config, B, H, W, C, F, R, Sx, stride, V, d, nnzb),
+        "config": {"workload": "%s: sparse Conv2D %s %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
+                               "nnzb=%d" % (args.config, "C-H-W-B / F-H-W-B, B x H x W x C =" if batch_first else "NHWC",
+                                            B, H, W, C, F, R, Sx, stride, V, d, nnzb),
                    "kernel": kernel, "timing": "events around %d back-to-back execs, operands resident" % args.steps},
         "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
         "reference_timing_loop": {"what": "11 warm-ups + 100 execs from an idle GPU (clock still ramping)",

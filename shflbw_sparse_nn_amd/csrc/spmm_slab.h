@@ -29,8 +29,8 @@ struct SpmmSlabCfg {
     static constexpr int NBUF = 8;           // batches a wave keeps in flight (even: the fragment sets alternate)
     static constexpr int FETCH_OPS = 3;      // loads per batch: two A fragments and a quad of offsets
     static constexpr int RID_REGS = 8;       // a wave's panels have at most RID_REGS * 64 rows
-    static constexpr int EPI_ROWB = 32 * 2 + 16;
-    static constexpr int EPI_WAVE_BYTES = 32 * EPI_ROWB;
+    static constexpr int EPI_ROWB = BN * 2 + 16;          // a staged row: all 64 columns and 16 bytes of padding
+    static constexpr int EPI_WAVE_BYTES = 16 * EPI_ROWB;  // 16 rows at a time
     static constexpr int LDS_MAX = 160 * 1024;
     // rows of B the LDS holds beside the row of zeros and the staging areas, rounded down to the 8 rows of a copy
     static constexpr int MAX_K = ((LDS_MAX - NW * EPI_WAVE_BYTES) / ROWB - 1) / 8 * 8;
@@ -67,9 +67,9 @@ __global__ void __launch_bounds__(SpmmSlabCfg::THREADS) spmm_shflbw_slab_kernel(
     // of offsets per pair and 64-slot group, 16 per batch
     const uint32_t pair32 = (uint32_t)(((lane >> 5) * 4 + (li >> 2)) * 32);
     const uint32_t lane16 = (uint32_t)lane * 16;
-    // epilogue: a lane writes 4 columns of row lane % 32, reads 16-byte piece lane % 4 of row lane / 4
-    const uint32_t wr = epi + (lane & 31) * Cfg::EPI_ROWB + (lane >> 5) * 8;
-    const uint32_t rd = epi + (lane >> 2) * Cfg::EPI_ROWB + (lane & 3) * 16;
+    // epilogue: a lane writes 4 columns (per 32-column block) of row lane % 16, reads 16-byte piece lane % 8 of row lane / 8
+    const uint32_t wr = epi + (lane & 15) * Cfg::EPI_ROWB + (lane >> 5) * 8;
+    const uint32_t rd = epi + (lane >> 3) * Cfg::EPI_ROWB + (lane & 7) * 16;
     const float alpha = a.alpha, beta = a.beta;
 
     struct Batch {
@@ -125,28 +125,43 @@ __global__ void __launch_bounds__(SpmmSlabCfg::THREADS) spmm_shflbw_slab_kernel(
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[nb][i] = 0.f;
         };
-        // fp32 -> fp16 (one rounding) -> staging area -> 16-byte pieces of 64-byte row segments -> rows of D
+        // fp32 -> fp16 (one rounding) -> staging area, 16 rows of all 64 columns at a time -> rows of D, eight lanes
+        // to a row: every store instruction writes whole 128-byte lines (half lines, written at different times,
+        // cost 1.4 x the bytes at the memory side with streaming stores)
         auto epilogue = [&]() __attribute__((always_inline)) {
             const int i0 = (p - pa) * V; // first row of the panel among the wave's rows
             int rid = ridreg[0];
 #pragma unroll
             for (int q = 1; q < Cfg::RID_REGS; q++) rid = (i0 >> 6) == q ? ridreg[q] : rid;
-            size_t roff[2];
+            const int col = n0 + (lane & 7) * 8;
 #pragma unroll
-            for (int it = 0; it < 2; it++) roff[it] = (size_t)__shfl(rid, (i0 & 63) + it * 16 + (lane >> 2)) * a.ldd;
+            for (int hh = 0; hh < 2; hh++) { // rows 16 hh .. 16 hh + 15: held by the lanes with bit 4 equal to hh
+                size_t roff[2];
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
+                for (int it = 0; it < 2; it++)
+                    roff[it] = (size_t)__shfl(rid, (i0 & 63) + hh * 16 + it * 8 + (lane >> 3)) * a.ldd;
+                if (((lane >> 4) & 1) == hh) {
 #pragma unroll
-                for (int ig = 0; ig < 4; ig++) {
-                    half4_t h;
+                    for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) h[e] = (half_t)(acc[nb][ig * 4 + e] * alpha);
-                    *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + ig * 16) = h;
+                        for (int ig = 0; ig < 4; ig++) {
+                            half4_t h;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) h[e] = (half_t)(acc[nb][ig * 4 + e] * alpha);
+                            *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + nb * 64 + ig * 16) = h;
+                        }
                 }
+                // Lanes exchange data through the staging area.  For the compiler every lane is a thread of its own: it
+                // may run the lanes that do not write through their reads first unless the wave is told to meet here.
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 half8_t v[2];
 #pragma unroll
-                for (int it = 0; it < 2; it++) v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * 16 * Cfg::EPI_ROWB);
-                const int col = n0 + nb * 32 + (lane & 3) * 8;
+                for (int it = 0; it < 2; it++) v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rd + it * 8 * Cfg::EPI_ROWB);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier(); // the next 16 rows overwrite what other lanes have just read
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 if (col < N) {
                     if (beta != 0.f) {
 #pragma unroll

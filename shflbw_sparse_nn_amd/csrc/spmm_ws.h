@@ -321,6 +321,11 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
                     }
                     // all loads (LDS pieces, C when used), then all stores: the vector-memory
                     // counter is in-order, a load issued behind a store would wait for the store
+                    if constexpr (ER != 32) { // only half of the lanes wrote: the wave meets before any lane reads
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    }
                     half8_t v[NIT], c[NIT];
 #pragma unroll
                     for (int it = 0; it < NIT; it++)

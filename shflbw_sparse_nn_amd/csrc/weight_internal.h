@@ -75,7 +75,7 @@ inline int mfma_kstep(int brow) { return brow >= 32 ? 16 : 32; }
 // Geometry of the slab form of the SpMM: a workgroup holds up to SLAB_MAX_K rows of SLAB_ROW_BYTES bytes (64 columns)
 // of B in LDS, one more row of zeros behind them (rounded up to a multiple of 8 rows) for the padding slots.
 constexpr int SLAB_ROW_BYTES = 128;
-constexpr int SLAB_MAX_K = 1112;
+constexpr int SLAB_MAX_K = 1128;
 // LDS byte offset of what slot id `k` of a weight with `ncol` columns reads: the start of slab row k with the XOR key
 // of the row, (k / 2) % 4, in the position of the 32-byte unit; padding slots (k < 0) read the row of zeros.
 inline int slab_row_offset(int k, int ncol)

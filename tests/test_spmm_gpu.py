@@ -183,7 +183,7 @@ def _slab_variant(V):
     (2048, 1024, 777, 32, 0.15, False),   # K not a multiple of 8: filler rows between the last row and the zeros
     (64, 64, 8, 32, 1.0, True),           # one column tile, two panels, one step each
     (256, 24000, 96, 32, 0.5, True),      # more column tiles than compute units: workgroups refill the slab
-    (8192, 128, 1112, 32, 0.05, True),    # the largest K the LDS takes; 256 panels over two column tiles
+    (8192, 128, 1128, 32, 0.05, True),    # the largest K the LDS takes; 256 panels over two column tiles
     (4096, 512, 512, 32, 0.02, True),     # about ten kept vectors a panel: groups with one to three steps, empty panels
     (96, 8, 40, 32, 0.6, True),           # N smaller than a piece of the second 32-column block
 ])

@@ -45,6 +45,13 @@ def conv_oracle(w, R, S, Cc, x_nhwc, stride, nthreads=0):
                                    w["row_permute_ids"], Bn, H, W, stride, R // 2, S // 2, x_nhwc, nthreads)
 
 
+def conv_oracle_batch_first(w, R, S, Cc, x_chwb, stride):
+    """The reference's loop nest on its own tensors: C-H-W-B in, F-H-W-B out, H and W bounding both."""
+    _, H, W, Bn = x_chwb.shape
+    return O.spconv_reference_chwb(w["nrow"], R, S, Cc, w["brow"], 1, w["indptr"], w["indices"], w["values"],
+                                   w["row_permute_ids"], Bn, H, W, stride, x_chwb)
+
+
 def abs_products_bound(w, B):
     """sum_k |a_k * b_k| per output element (fp32): the scale against which fp32 summation
     order differences are measured."""
@@ -64,6 +71,10 @@ CONV_CONFIGS = {
                  x_dist=("normal", 1.0)),
     "cfg4": dict(B=32, H=28, W=28, C=256, F=512, R=3, S=3, stride=2, V=32, d=0.3, w_dist=("normal", 0.05),
                  x_dist=("normal", 1.0)),
+    # the reference's own test case on its own tensors (test/test.spconv.blockwise.cu:10-14: 128 x 14 x 14 x 256 -> 256,
+    # 3 x 3, density 0.1): C-H-W-B input, F-H-W-B output, not one of the graded configurations
+    "refconv": dict(B=128, H=14, W=14, C=256, F=256, R=3, S=3, stride=1, V=64, d=0.1, w_dist=("normal", 0.05),
+                    x_dist=("normal", 1.0), layout="chwb"),
 }
 
 
