@@ -61,3 +61,32 @@ def test_spconv_exec_in_a_graph(torch_gpu, variant):
     op = S.SpconvBlockwiseOp(variant)
     op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr())
     _replays(torch, op, [to_dev(torch, x) for x in xs], dX, dY, refs)
+
+
+def test_slab_spmm_exec_in_a_graph(torch_gpu):
+    torch = torch_gpu
+    M, K, N, V = 1024, 520, 264, 32  # block height 32, few columns: the variant that keeps a slab of B in LDS
+    w = P.make_weight(M, K, V, 0.2, True, 2021, integer=True)
+    Bs = [P.make_dense(K, N, 2021 + i, integer=True) for i in range(2)]
+    refs = [O.float_to_half(P.spmm_oracle(w, B)) for B in Bs]
+    m = upload_weight(w)
+    dB = torch.empty((K, N), dtype=torch.float16, device="cuda")
+    dD = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    slab = [i for i, n in enumerate(S.spmm_variants(V)) if n.startswith("slab")][0]
+    op = S.SpmmBlockwiseOp(slab)
+    op.initialize(m, N, dB.data_ptr(), dD.data_ptr())
+    _replays(torch, op, [to_dev(torch, B) for B in Bs], dB, dD, refs)
+
+
+def test_reference_layout_spconv_exec_in_a_graph(torch_gpu):
+    torch = torch_gpu
+    Bn, H, W, C, F, R, Sx, stride, V = 8, 7, 7, 32, 64, 3, 3, 1, 32
+    w = P.make_weight(F, R * Sx * C, V, 0.3, True, 2021, integer=True)
+    xs = [np.random.default_rng(5 + i).integers(-4, 5, size=(C, H, W, Bn)).astype(np.float16) for i in range(2)]
+    refs = [O.float_to_half(P.conv_oracle_batch_first(w, R, Sx, C, x, stride)) for x in xs]
+    f = upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
+    dX = torch.empty((C, H, W, Bn), dtype=torch.float16, device="cuda")
+    dY = torch.empty(refs[0].shape, dtype=torch.float16, device="cuda")
+    op = S.SpconvBlockwiseOp()
+    op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr(), batch_innermost=True)
+    _replays(torch, op, [to_dev(torch, x) for x in xs], dX, dY, refs)
