@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Benchmark of the Shfl-BW hot path on one MI355X.  Default workload: the headline SpMM, M = K = N = 4096,
-block size 64, density 0.1, row-permuted (BASELINE.json configs[1]).
+block size 64, density 0.1, row-permuted (the graded headline configuration, cfg1).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg0|cfg1|cfg2|cfg3|cfg4|refconv]
 
