@@ -119,17 +119,21 @@ static bool spmm_variant_offsets32(const SpmmVariant* v) { return v && v->name[0
 // there, 5-20 % slower once the wide tiles fill the chip).
 // Block height 32 and at most SLAB_MAX_K columns: the slab variant moves less data between the L2 and the
 // compute units once a workgroup runs enough kept vectors over the 128 KiB slab it has to load first.  Taken
-// when a workgroup's panels keep at least 6 vectors per column of A on average (below that the slab load
-// dominates: measured 7-30 % slower at 1.6) and A has at least 512 columns (with fewer, B fits the L2 and
-// the gathers of the role-split kernel all hit) and the packed A is at most 5 MB (all workgroups of an XCD
-// stream all of A from its 4 MB L2; at 6.7 MB the variant was 25 % slower).  Measured 2-28 % faster inside
-// these bounds (M = 4096, K = 1024, N = 4096, density 0.2: 15.1 against 16.5 us).
+// when (34 shapes measured with both kernels, each pair on one box)
+//  * a workgroup's panels keep at least 3 vectors per column of A on average (3.2: 5 % faster, 2.4: 5-20 %
+//    slower, 1.6: equal to 30 % slower: the slab load is not paid back),
+//  * A has at least 384 columns (at 256 B fits the L2, the gathers of the role-split kernel all hit, and the
+//    two kernels tie),
+//  * there are at least 32 column tiles, so that four or more workgroups of an XCD stream the same chunk of A
+//    at the same time and share it in their L2 (16 tiles: 15 % slower).
+// Inside these bounds: equal to 28 % faster (M = 4096, K = 1024, N = 4096, density 0.2: 15.1 against 16.5 us;
+// M = 8192, density 0.3: 31.3 against 38.7 us).
 static int auto_spmm_variant(const shflbw_weight* w, int N)
 {
     const int brow = w->brow, X = w->nrow / w->brow;
     int count = 0;
     const SpmmVariant* all = spmm_variants(&count);
-    if (brow == 32 && !w->packed_slab.empty() && w->ncol >= 512 && X > 0) {
+    if (brow == 32 && !w->packed_slab.empty() && w->ncol >= 384 && X > 0) {
         int seen = 0;
         for (int i = 0; i < count; i++) {
             if (all[i].V != brow) continue;
@@ -139,7 +143,7 @@ static int auto_spmm_variant(const shflbw_weight* w, int N)
                 const int chunks = std::max(1, std::min(X, cus / n_tiles)); // as the launcher deals the panels
                 const double panels_per_wg = (double)X / chunks;
                 const double vectors_per_column = panels_per_wg * w->nnzb / ((double)X * w->ncol);
-                if (vectors_per_column >= 6.0 && (double)w->nnzb * brow * 2 <= 5.0e6) return seen;
+                if (vectors_per_column >= 3.0 && n_tiles >= 32) return seen;
             }
             seen++;
         }
