@@ -177,3 +177,31 @@ def test_reference_layout_needs_a_batch_of_eights(torch_gpu):
     with pytest.raises(capi.ShflbwError) as e:
         Sx.SpconvBlockwiseOp().initialize(f, 4, 5, 5, 1, t.data_ptr(), t.data_ptr(), batch_innermost=True)
     assert e.value.status == capi.ERR_SHAPE
+
+
+def test_reference_layout_seeded_random_shapes(torch_gpu):
+    """Twenty small seeded problems on the reference's tensors: filter extents 1..5, strides 1..3, batches of 8..32."""
+    import shflbw_sparse_nn_amd as Sx
+    torch = torch_gpu
+    rng = np.random.default_rng(777)
+    for case in range(20):
+        V = int(rng.choice([16, 32, 64, 128]))
+        F = V * int(rng.integers(1, 4))
+        C = int(rng.integers(1, 24))
+        R, S_ = int(rng.choice([1, 3, 5])), int(rng.choice([1, 2, 3, 5]))
+        H, W = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        Bn = 8 * int(rng.integers(1, 5))
+        stride = int(rng.integers(1, 4))
+        d = float(rng.choice([0.1, 0.4, 1.0]))
+        print("case", case, (Bn, H, W, C, F, R, S_, stride, V, d), flush=True)
+        w = P.make_weight(F, R * S_ * C, V, d, bool(rng.integers(0, 2)), 300 + case, integer=True)
+        x = rng.integers(-4, 5, size=(C, H, W, Bn)).astype(np.float16)
+        ref = O.float_to_half(P.conv_oracle_batch_first(w, R, S_, C, x, stride))
+        f = P.upload_weight(w, R, S_, C, cls=Sx.BlockwiseSpFilter)
+        dX = P.to_dev(torch, x)
+        dY = torch.full((F, H, W, Bn), float("nan"), dtype=torch.float16, device="cuda")
+        op = Sx.SpconvBlockwiseOp()
+        op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr(), batch_innermost=True)
+        op(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)

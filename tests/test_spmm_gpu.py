@@ -221,3 +221,24 @@ def test_slab_variant_refuses_wide_weights(torch_gpu):
     with pytest.raises(capi.ShflbwError) as e:
         run_spmm(torch_gpu, w, B, variant=_slab_variant(32))
     assert e.value.status == capi.ERR_UNSUPPORTED
+
+
+def test_slab_variant_seeded_random_shapes(torch_gpu):
+    """Thirty small seeded shapes (ragged N, K not a multiple of 8, densities from nearly empty to full, permuted or
+    not, with and without C): every one bit-exact against the oracle."""
+    rng = np.random.default_rng(20211)
+    v = _slab_variant(32)
+    for case in range(30):
+        M = 32 * int(rng.integers(1, 20))
+        K = int(rng.integers(1, 400))
+        N = 8 * int(rng.integers(1, 60))
+        d = float(rng.choice([0.02, 0.1, 0.3, 0.6, 1.0]))
+        permute = bool(rng.integers(0, 2))
+        with_c = bool(rng.integers(0, 2))
+        print("case", case, (M, N, K, d, permute, with_c), flush=True)
+        w = P.make_weight(M, K, 32, d, permute, 100 + case, integer=True)
+        B = P.make_dense(K, N, 100 + case, integer=True)
+        Cm = P.make_dense(M, N, 100 + case, integer=True, stream=3) if with_c else None
+        got = run_spmm(torch_gpu, w, B, Cmat=Cm, variant=v)
+        ref = O.float_to_half(P.spmm_oracle(w, B, Cm, 1.0, 1.0) if with_c else P.spmm_oracle(w, B))
+        np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
