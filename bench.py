@@ -279,7 +279,7 @@ def bench_conv(args, np, torch, S, P):
         oracle = lambda w, x, **kw: P.conv_oracle_batch_first(w, R, Sx, C, x, stride)
     else:
         Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
-        in_shape, out_shape, variant = (B, H, W, C), (B, Ho, Wo, F), max(args.variant, 0)
+        in_shape, out_shape, variant = (B, H, W, C), (B, Ho, Wo, F), args.variant
         oracle = lambda w, x, **kw: P.conv_oracle(w, R, Sx, C, x, stride, **kw)
     npix = B * Ho * Wo
     stream = torch.cuda.current_stream()
@@ -334,7 +334,7 @@ def bench_conv(args, np, torch, S, P):
                                "the first %d panels" % XS, O.max_threads())
 
     eff_tflops = eff_flops / t / 1e12
-    kernel = S.spconv_variant_name(variant)
+    kernel = S.spconv_variant_name(op._state.variant)
     traffic = measured_traffic(args.config, kernel) if args.traffic is None else round(float(args.traffic))
     print(json.dumps({
         "metric": "effective sparse TFLOP/s + %% fp16 MFMA peak, SpConv2D %s" % args.config,

@@ -195,13 +195,17 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  * init allocates device scratch inside the filter object (freed with it; states made from one
  * filter with equal scratch size share it, so launch them on one stream); exec only launches, in
  * order on `stream`: a layout pass over the input, the SpMM kernel, and the transpose to NHWC.
- * shflbw_spconv_init_variant:
- *   variant 0 (default) = plane form: the input is rewritten once per call as channel-major padded
+ * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice, 5 when B % 8 == 0, else 0):
+ *   variant 0 = plane form: the input is rewritten once per call as channel-major padded
  *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
  *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,
  *     its address generation is the per-id offset of the gather;
  *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads);
- *   variant 2 = explicit im2col matrix, SpMM, transpose.
+ *   variant 2 = explicit im2col matrix, SpMM, transpose;
+ *   variant 3 = the steps of variant 0 in one persistent launch;
+ *   variant 5 = plane form with the batch innermost in the planes and in the filter-major result (B % 8 == 0):
+ *     every tap offset is then a multiple of 16 bytes, one copy of the planes serves all taps, and the result
+ *     holds output pixels only.
  * ------------------------------------------------------------------------- */
 typedef struct shflbw_spconv_state {
     size_t shared_mem_size;
@@ -229,7 +233,10 @@ typedef struct shflbw_spconv_state {
      * [plane_copies][stride*stride][C][plane_pitch]; a "pixel" of the GEMM is a position
      * b*plane_rows*plane_cols + i*plane_cols + j of that padded grid, np = B*plane_rows*plane_cols of
      * them, and result_fm is [F][np].  im2col form (variant 2): im2col is the matrix [R*S*C][np],
-     * np = B*Ho*Wo rounded up to 64, result_fm [F][np]. */
+     * np = B*Ho*Wo rounded up to 64, result_fm [F][np].  Batch-innermost forms (variants 4, 5): `planes` is
+     * [stride*stride][C][plane_pitch] with position (i*plane_cols + j)*B + b, plane_rows = Ho + (R-1)/stride,
+     * plane_cols = Wo + (S-1)/stride; ncols = Ho*plane_cols*B columns of the GEMM; result_fm (variant 5) is
+     * [F][Ho*Wo*B]. */
     void* im2col;
     void* result_fm;
     int np;

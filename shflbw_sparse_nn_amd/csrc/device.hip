@@ -384,7 +384,7 @@ int shflbw_spmm_exec(const shflbw_spmm_state* state, void* stream)
 int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
                        const void* IFMap, void* OFMap)
 {
-    return shflbw_spconv_init_variant(state, f, B, H, W, stride, IFMap, OFMap, 0);
+    return shflbw_spconv_init_variant(state, f, B, H, W, stride, IFMap, OFMap, -1);
 }
 
 // Argument checks of a convolution and every field of the state that does not depend on device scratch.
@@ -514,6 +514,9 @@ static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, c
     return SHFLBW_OK;
 }
 
+static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                             const void* IFMap, void* OFMap, int variant);
+
 int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
                                const void* IFMap, void* OFMap, int variant)
 {
@@ -522,6 +525,10 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         set_error("spconv_init: form 4 works on C-H-W-B / F-H-W-B tensors; call shflbw_spconv_init_chwb");
         return SHFLBW_ERR_INVALID;
     }
+    // the library's choice: the batch-innermost plane form where the batch allows it (one copy of the planes instead
+    // of two, no dead plane rows in the result: cfg3 22.9 against 25.3 us, cfg4 24.0 against 25.9), else the plane form
+    if (variant < 0) variant = B > 0 && B % 8 == 0 ? 5 : 0;
+    if (variant == 5) return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, 5);
     int frc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
     if (frc != SHFLBW_OK) return frc;
     const int Ho = state->Ho, Wo = state->Wo;
@@ -628,51 +635,63 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
     return SHFLBW_OK;
 }
 
-int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                            const void* IFMap, void* OFMap)
+// Forms 4 and 5: phase planes with the batch innermost, planes[phase (a, b)][c][(i * PW + j) * B + img] =
+// in(i * stride + a - R/2, j * stride + b - S/2) of image img and channel c, PHX = Ho + (R-1)/stride rows and
+// PW = Wo + (S-1)/stride columns.  Every tap offset is a multiple of B values, 16 bytes or more: one copy of the
+// planes serves all taps.  The SpMM runs over the Ho * PW * B columns (ho, j, img) of the padded output grid and
+// drops the padding columns in its epilogue (output_column()).
+//   form 4: the caller's tensors are C-H-W-B / F-H-W-B (the reference's), H and W bound input and output alike,
+//           the SpMM writes OFMap itself;
+//   form 5: the caller's tensors are NHWC with true stride and padding; the SpMM writes result_fm[f][(ho, wo, img)],
+//           a tile transpose writes OFMap.
+static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                             const void* IFMap, void* OFMap, int variant)
 {
-    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, 4);
+    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
     if (rc != SHFLBW_OK) return rc;
-    if (B % 8 != 0) { // the reference's kernel moves 8 batch entries at a time (spconv/blockwise_kernel.h:200-207)
-        set_error("spconv_init_chwb: the batch must be a multiple of 8 (got %d)", B);
+    if (B % 8 != 0) { // the reference's kernel moves 8 batch entries at a time too (spconv/blockwise_kernel.h:200-207)
+        set_error("spconv_init: the batch must be a multiple of 8 for this form (got %d)", B);
         return SHFLBW_ERR_SHAPE;
     }
     const ConvChwbKernel* k = conv_chwb_kernel(f->brow);
     if (!k) {
-        set_error("spconv_init_chwb: no kernel for block size %d", f->brow);
+        set_error("spconv_init: no kernel for block size %d", f->brow);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     SHFLBW_HIP_TRY(k->prepare());
-    // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
-    state->Ho = H;
-    state->Wo = W;
-    const int s = stride;
-    const long PHX = H + (f->R - 1) / s, PW = W + (f->S - 1) / s;
+    if (variant == 4) { // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
+        state->Ho = H;
+        state->Wo = W;
+    }
+    const int s = stride, Ho = state->Ho, Wo = state->Wo;
+    const long PHX = Ho + (f->R - 1) / s, PW = Wo + (f->S - 1) / s;
     const long np = PHX * PW * B;                                  // values of one channel plane
     const long pitch = (np + (long)((f->S - 1) / s) * B + 8 + 63) / 64 * 64;
     const long rows = (long)s * s * f->C;
-    const long ncols = (long)H * PW * B;                           // columns of the GEMM: the padded output grid
+    const long ncols = (long)Ho * PW * B;                          // columns of the GEMM: the padded output grid
     if (ncols > 0x7fffffffL || (unsigned long long)(rows + 1) * (unsigned long long)pitch * 2ull > 0xffffffffull) {
-        set_error("spconv_init_chwb: problem too large (%ld channel rows of %ld values)", rows, pitch);
+        set_error("spconv_init: problem too large (%ld channel rows of %ld values)", rows, pitch);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
     const size_t slots = f->packed_indices.size();
     const size_t planes_bytes = up256((size_t)(rows + 1) * pitch * 2), ids_bytes = up256(slots * sizeof(int) + 64);
+    const size_t dm_bytes = variant == 5 ? up256((size_t)f->F * Ho * Wo * B * 2) : 0;
+    const size_t total = planes_bytes + dm_bytes + 2 * ids_bytes;
     shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is bookkeeping of the handle (see shflbw_spconv_init_variant)
     std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
     char* scratch = nullptr;
-    const int key[5] = {4, B, H, W, stride};
+    const int key[5] = {variant, B, H, W, stride};
     for (auto& sc : fw->conv_scratch)
-        if (sc.bytes == planes_bytes + 2 * ids_bytes && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap)
+        if (sc.bytes == total && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap)
             scratch = (char*)sc.ptr;
     if (!scratch) {
         void* ptr = nullptr;
-        if (hipMalloc(&ptr, planes_bytes + 2 * ids_bytes) != hipSuccess) {
-            set_error("spconv_init_chwb: cannot allocate %zu bytes of device scratch", planes_bytes + 2 * ids_bytes);
+        if (hipMalloc(&ptr, total) != hipSuccess) {
+            set_error("spconv_init: cannot allocate %zu bytes of device scratch", total);
             return SHFLBW_ERR_HIP;
         }
-        fw->conv_scratch.push_back(shflbw_weight::Scratch{planes_bytes + 2 * ids_bytes, ptr, {4, B, H, W, stride}, IFMap, OFMap});
+        fw->conv_scratch.push_back(shflbw_weight::Scratch{total, ptr, {variant, B, H, W, stride}, IFMap, OFMap});
         scratch = (char*)ptr;
         SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes)); // includes the row of zeros behind the last channel row
         // kept-column id k = (r*S + t)*C + c  ->  element offset of the (phase, channel) row + tap offset
@@ -691,21 +710,24 @@ int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, 
             const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
             ids_pm[grp * 64 + 16 * p + 4 * j + r] = ids[q];
         }
-        SHFLBW_HIP_TRY(hipMemcpy(scratch + planes_bytes, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
-        SHFLBW_HIP_TRY(hipMemcpy(scratch + planes_bytes + ids_bytes, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+        char* ids_dev = scratch + planes_bytes + dm_bytes;
+        SHFLBW_HIP_TRY(hipMemcpy(ids_dev, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
+        SHFLBW_HIP_TRY(hipMemcpy(ids_dev + ids_bytes, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
     }
     state->planes = scratch;
+    state->result_fm = variant == 5 ? scratch + planes_bytes : nullptr;
     state->np = (int)np;
     state->plane_rows = (int)PHX;
     state->plane_cols = (int)PW;
     state->plane_pitch = (int)pitch;
     state->plane_copies = 1;
     state->ncols = (int)ncols;
-    // the SpMM in the middle writes the output tensor itself: row f of the result is the F-H-W-B row of filter f
-    rc = shflbw_spmm_init_variant(&state->spmm, f, (int)ncols, state->planes, nullptr, OFMap, 1.f, 0.f, 0);
+    // the SpMM in the middle: row f of its result is the row of filter f, in OFMap itself (form 4) or in result_fm
+    rc = shflbw_spmm_init_variant(&state->spmm, f, (int)ncols, state->planes, nullptr,
+                                  variant == 5 ? state->result_fm : OFMap, 1.f, 0.f, 0);
     if (rc != SHFLBW_OK) return rc;
-    state->spmm.packed_indices = (const int*)(scratch + planes_bytes);
-    state->spmm.packed_indices_pm = (const int*)(scratch + planes_bytes + ids_bytes);
+    state->spmm.packed_indices = (const int*)(scratch + planes_bytes + dm_bytes);
+    state->spmm.packed_indices_pm = (const int*)(scratch + planes_bytes + dm_bytes + ids_bytes);
     state->spmm.ldb_bytes = 2;
     state->spmm.args.K = (int)((rows + 1) * pitch);
     state->shared_mem_size = (size_t)k->lds_bytes;
@@ -715,6 +737,12 @@ int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, 
     state->block_dim[1] = state->block_dim[2] = 1;
     state->init_success = 1;
     return SHFLBW_OK;
+}
+
+int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                            const void* IFMap, void* OFMap)
+{
+    return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, 4);
 }
 
 int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
@@ -746,19 +774,26 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
-    if (state->variant == 4) {
+    if (state->variant == 4 || state->variant == 5) {
         const ConvChwbKernel* k = conv_chwb_kernel(state->brow);
         if (!k) return SHFLBW_ERR_UNSUPPORTED;
-        hipError_t e = launch_chwb_to_planes(a.in, (half_t*)state->planes, a.B, a.H, a.W, a.C, a.R, a.S, a.stride,
-                                             state->plane_rows, state->plane_cols, state->plane_pitch, (hipStream_t)stream);
+        const bool nhwc = state->variant == 5;
+        hipError_t e = nhwc ? launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
+                                                    state->plane_pitch, 1, (hipStream_t)stream, 1)
+                            : launch_chwb_to_planes(a.in, (half_t*)state->planes, a.B, a.H, a.W, a.C, a.R, a.S, a.stride,
+                                                    state->plane_rows, state->plane_cols, state->plane_pitch,
+                                                    (hipStream_t)stream);
         SpmmLaunchArgs m;
         fill_spmm_launch_args(&state->spmm, k->BN, &m);
         m.alternate = 0;
-        m.ldd = a.H * a.W * a.B;                    // a row of the output: one filter, H x W x B values
+        m.ldd = a.Ho * a.Wo * a.B;                  // a row of the result: one filter, Ho x Wo x B values
         m.dmap_row = state->plane_cols * a.B;       // columns of the GEMM per row of the padded output grid
-        m.dmap_valid = a.W * a.B;                   // ... of which the first W x B are output values
+        m.dmap_valid = a.Wo * a.B;                  // ... of which the first Wo x B are output values
         m.dmap_magic = udiv_magic(m.dmap_row);
         if (e == hipSuccess && m.X > 0) e = k->launch(m, (hipStream_t)stream);
+        if (e == hipSuccess && nhwc) // result_fm[f][(ho, wo, img)] -> OFMap[img][ho][wo][f]
+            e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, a.Ho * a.Wo * a.B, a.B, a.Ho, a.Wo,
+                                      a.Ho, a.Wo, (hipStream_t)stream, 1);
         if (e != hipSuccess) {
             set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));
             return SHFLBW_ERR_HIP;
@@ -949,6 +984,7 @@ static const char* const g_spconv_forms[] = {
     "im2col+spmm+transpose",  // 2: explicit im2col matrix, three launches
     "fused-planes",           // 3: the steps of form 0 in one persistent launch
     "chwb-planes+spmm",       // 4: the reference's batch-innermost tensors (shflbw_spconv_init_chwb only): padded copy, SpMM
+    "bplanes+spmm+transpose", // 5: NHWC tensors, planes and result with the batch innermost (batch a multiple of 8): three launches
 };
 
 int shflbw_spconv_variant_count(void) { return (int)(sizeof(g_spconv_forms) / sizeof(g_spconv_forms[0])); }

@@ -304,10 +304,10 @@ __global__ void __launch_bounds__(256) nhwc_to_planes_kernel(const half_t* __res
         [&](int i, int j) { // source row = position p0 + i (+ copy), piece = channels c0 + 8j ..
             half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
             const int n = p0 + i + copy;
-            const int img = n / PS, rem = n % PS;
+            const int img = g.batch_inner ? n % g.B : n / PS, rem = g.batch_inner ? n / g.B : n % PS;
             const int hi = (rem / g.PW) * g.stride + pa - g.pad_h, wi = (rem % g.PW) * g.stride + pb - g.pad_w;
             const int c = c0 + j * 8;
-            if (img < g.B && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && c < g.C)
+            if (img < g.B && rem < PS && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && c < g.C)
                 v = *(const half8_t*)(in + ((size_t)(img * g.H + hi) * g.W + wi) * g.C + c);
             return v;
         },
@@ -318,7 +318,7 @@ __global__ void __launch_bounds__(256) nhwc_to_planes_kernel(const half_t* __res
 
 // grid: (position tiles, filter tiles); block 256.  dm has rows of NP values.
 __global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __restrict__ dm, half_t* __restrict__ out, int F,
-                                                             int NP, int B, int PH, int PW, int Ho, int Wo)
+                                                             int NP, int B, int PH, int PW, int Ho, int Wo, int batch_inner)
 {
     __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
     const int p0 = blockIdx.x * TT, f0 = blockIdx.y * TT;
@@ -332,7 +332,7 @@ __global__ void __launch_bounds__(256) planes_to_nhwc_kernel(const half_t* __res
         },
         [&](int o, int q, half8_t v) { // destination row = the pixel at position p0 + o, filters f0 + 8q ..
             const int n = p0 + o, f = f0 + q * 8;
-            const int img = n / PS, rem = n % PS, ho = rem / PW, wo = rem % PW;
+            const int img = batch_inner ? n % B : n / PS, rem = batch_inner ? n / B : n % PS, ho = rem / PW, wo = rem % PW;
             // streaming store: the output is not read again here and should not push the next launch's input out of the caches
             if (img < B && ho < Ho && wo < Wo && f < F)
                 __builtin_nontemporal_store(v, (half8_t*)(out + ((size_t)(img * Ho + ho) * Wo + wo) * F + f));
@@ -676,9 +676,9 @@ hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, i
 }
 
 hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int PH, int PW, int pitch, int copies,
-                                 hipStream_t stream)
+                                 hipStream_t stream, int batch_inner)
 {
-    PlaneGeom g{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, PH, PW, pitch, copies, 0, {}};
+    PlaneGeom g{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, PH, PW, pitch, copies, 0, {}, batch_inner};
     if (!fill_wanted_planes(g, a.R, a.S)) return hipErrorInvalidValue;
     const int np = a.B * PH * PW;
     const dim3 grid((np + TT - 1) / TT, (a.C + TT - 1) / TT, g.nwanted);
@@ -687,10 +687,10 @@ hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int 
 }
 
 hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, int B, int PH, int PW, int Ho, int Wo,
-                                 hipStream_t stream)
+                                 hipStream_t stream, int batch_inner)
 {
     const dim3 grid((NP + TT - 1) / TT, (F + TT - 1) / TT);
-    hipLaunchKernelGGL(planes_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, NP, B, PH, PW, Ho, Wo);
+    hipLaunchKernelGGL(planes_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, NP, B, PH, PW, Ho, Wo, batch_inner);
     return hipGetLastError();
 }
 

@@ -38,6 +38,7 @@ struct PlaneGeom {
     int copies;   // 1, or 2 with the copy moved by one value
     int nwanted;  // (copy, phase) planes some tap reads; the others are never written
     unsigned char wanted[32]; // copy * stride * stride + phase of each
+    int batch_inner; // position n of a plane is (i * PW + j) * B + img instead of (img * PH + i) * PW + j
 };
 
 bool fill_wanted_planes(PlaneGeom& g, int R, int S);
@@ -94,10 +95,11 @@ const ConvChwbKernel* conv_chwb_kernel(int V);
 // Stages 1 and 3 of the plane form of the convolution: NHWC input -> channel-major padded planes (one per
 // stride phase, `copies` = 1 or 2 with a copy moved by one value, rows of `pitch` values), and the
 // filter-major result over plane positions (rows of NP values) -> NHWC output.
+// batch_inner: the positions of a plane (and of the result) run (row, column, image) instead of (image, row, column)
 hipError_t launch_nhwc_to_planes(const SpconvLaunchArgs& a, half_t* planes, int PH, int PW, int pitch, int copies,
-                                 hipStream_t stream);
+                                 hipStream_t stream, int batch_inner = 0);
 hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, int B, int PH, int PW, int Ho, int Wo,
-                                 hipStream_t stream);
+                                 hipStream_t stream, int batch_inner = 0);
 
 // Plane-form ids computed on the device (for callers that may not copy from the host): slot-ordered and
 // producer-major element offsets from the packed kept-column ids; padding slots get `zero_id`, the offset of a

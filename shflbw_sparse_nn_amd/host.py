@@ -205,9 +205,9 @@ class SpmmBlockwiseOp:
 
 class SpconvBlockwiseOp:
     """initialize(spfilter, B, H, W, stride, IFMap, OFMap); NHWC tensors, H and W are input extents.
-    `variant` selects the form of the convolution (spconv_variants() names them); 0 is the library's default."""
+    `variant` selects the form of the convolution (spconv_variants() names them); -1 is the library's choice."""
 
-    def __init__(self, variant=0):
+    def __init__(self, variant=-1):
         self._lib = capi.load()
         self._state = capi.SpconvState()
         self._variant = variant

@@ -19,8 +19,12 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    # 0: plane layout + SpMM + transpose (default), 1: one direct kernel, 2: im2col matrix + SpMM + transpose, 3: form 0 fused into one launch
-    for variant in ((0, 3, 1, 2) if V != 16 else (0, 3, 2)):
+    # 0: plane layout + SpMM + transpose, 1: one direct kernel, 2: im2col matrix + SpMM + transpose, 3: form 0 fused into
+    # one launch, 5: planes and result with the batch innermost (batches that are multiples of 8)
+    forms = (0, 3, 1, 2) if V != 16 else (0, 3, 2)
+    if Bn % 8 == 0:
+        forms += (5,)
+    for variant in forms:
         print("conv", (Bn, H, W, C, F, R, S, stride, V, d, permute), "form", variant, flush=True)
         got = run_spconv(torch, w, R, S, C, x, stride, variant)
         assert got.shape == ref.shape
@@ -38,6 +42,12 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     (2, 12, 10, 8, 64, 5, 5, 2, 32, 0.3, True),   # 5x5 stride 2: tap offsets 0..2 inside a phase plane
     (1, 11, 9, 16, 64, 3, 3, 3, 64, 0.5, True),   # stride 3: nine phase planes, one tap each
     (2, 6, 20, 8, 32, 1, 7, 1, 32, 0.4, True),    # 1x7 filter: seven tap offsets in one row
+    # batches that are multiples of 8: the batch-innermost form runs too
+    (8, 7, 6, 16, 64, 3, 3, 2, 64, 0.3, True),    # stride 2, odd extents
+    (8, 5, 9, 8, 32, 5, 3, 1, 32, 0.4, False),    # rectangular filter, no permutation
+    (24, 6, 5, 24, 48, 3, 3, 3, 16, 0.5, True),   # stride 3, block height 16, batch of 24
+    (16, 4, 4, 8, 128, 1, 1, 1, 128, 0.6, True),  # 1x1 filter: no padding at all
+    (8, 9, 8, 16, 64, 4, 2, 2, 32, 0.3, True),    # even filter extents: the output is larger than input / stride
 ])
 def test_exact_shapes(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute):
     _exact(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute)
@@ -136,6 +146,13 @@ def test_non_finite_input_does_not_leak_through_padding(torch_gpu):
         assert np.array_equal(np.isnan(got), np.isnan(ref)), "form %d: NaN pattern differs" % variant
         ok = ~np.isnan(ref)
         np.testing.assert_array_equal(got[ok], ref[ok], err_msg="form %d" % variant)
+    # the batch-innermost form needs a batch of eights: the same two images four times over
+    x8 = np.concatenate([x] * 4)
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref8 = O.float_to_half(P.conv_oracle(w, R, Sx, C, x8, stride))
+    got = run_spconv(torch_gpu, w, R, Sx, C, x8, stride, 5)
+    assert np.array_equal(np.isnan(got), np.isnan(ref8)), "form 5: NaN pattern differs"
+    np.testing.assert_array_equal(got[~np.isnan(ref8)], ref8[~np.isnan(ref8)], err_msg="form 5")
 
 
 @pytest.mark.parametrize("Bn,H,W,C,F,R,S,stride,V,d,permute", [
@@ -205,3 +222,12 @@ def test_reference_layout_seeded_random_shapes(torch_gpu):
         op(torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
+
+
+def test_batch_innermost_form_needs_a_batch_of_eights(torch_gpu):
+    from shflbw_sparse_nn_amd import capi
+    w = P.make_weight(64, 9 * 8, 32, 0.3, True, 3, integer=True)
+    x = np.zeros((4, 5, 5, 8), dtype=np.float16)
+    with pytest.raises(capi.ShflbwError) as e:
+        run_spconv(torch_gpu, w, 3, 3, 8, x, 1, 5)
+    assert e.value.status == capi.ERR_SHAPE

@@ -121,7 +121,7 @@ def run_spmm(torch, w, B, Cmat=None, alpha=1.0, beta=None, variant=-1, poison=Tr
     return dD.cpu().numpy()
 
 
-def run_spconv(torch, w, R, Sx, Cc, x_nhwc, stride, variant=0):
+def run_spconv(torch, w, R, Sx, Cc, x_nhwc, stride, variant=-1):
     f = upload_weight(w, R, Sx, Cc, cls=_S().BlockwiseSpFilter)
     Bn, H, W, _ = x_nhwc.shape
     dX = to_dev(torch, x_nhwc)
