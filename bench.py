@@ -1,19 +1,28 @@
 #!/usr/bin/env python3
-"""Benchmark of the Shfl-BW hot path on one MI355X.  Default workload: the headline SpMM, M = K = N = 4096,
-block size 64, density 0.1, row-permuted (the graded headline configuration, cfg1).
+"""Benchmark of the Shfl-BW hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg0|cfg1|cfg2|cfg3|cfg4|refconv]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config all|cfg0|cfg1|cfg2|cfg3|cfg4|refconv]
 
-A step is one `exec` of the operator on device-resident operands (fp16 in, fp32 accumulate, fp16 out):
-one launch for the SpMM configs (cfg0-cfg2), the whole convolution for cfg3/cfg4.  Timing follows the
-reference's benchmark (benchmark/benchmark.spmm.cu:29-50, benchmark.spconv.cu:29-50): warm-up launches,
-then K back-to-back launches between two events on the launch stream; mean per launch.  Prints one JSON
-line: effective sparse TFLOP/s (2 * nnzb * V * N / t), the roofline of the kernel, and the CPU oracle timed
-on the host cores as a baseline; the SpMM line also carries a dense fp16 GEMM of the same shape.
+Default (`--config all`): every graded configuration is measured - the SpMM configs cfg0, cfg1 (the headline:
+M = K = N = 4096, block size 64, density 0.1, row-permuted) and cfg2, the sparse Conv2D configs cfg3 and cfg4 - and
+ONE JSON line is printed: its top-level figures are the headline's, its `configs` array holds kernel, time,
+effective TFLOP/s, share of the fp16 MFMA peak and roofline of all five.  `--config <name>` measures one
+configuration alone (what the profiles under profiles/ were taken with) and prints its full line.
+
+A step is one `exec` of the operator on device-resident operands (fp16 in, fp32 accumulate, fp16 out): one launch
+for the SpMM configs, the whole convolution (every launch of the form the library chooses) for cfg3 / cfg4.  Every
+configuration first passes a correctness gate (bit-exact against the CPU oracle on the integer twin of the
+workload).  Timing follows the reference's benchmark (benchmark/benchmark.spmm.cu:29-50, benchmark.spconv.cu:29-50):
+W warm-up launches, then K back-to-back launches between two events on the launch stream - here WINDOWS such
+windows in a row; `ms_per_step` is the median window, the fastest and slowest are reported beside it (a single
+window of a few launches falls into the clock ramp of an idle GPU).  The line carries the roofline of the kernel and
+the CPU oracle timed on the host cores as a baseline (headline only); the headline also carries a dense fp16 GEMM of
+the same shape.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -23,6 +32,7 @@ if ROOT not in sys.path:
 
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix-core peak
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+WINDOWS = 5                    # timed windows of `steps` launches each; the median is the figure
 
 
 def measured_traffic(config, kernel):
@@ -60,13 +70,27 @@ def reference_loop(torch, stream, op):
     return time_launches(torch, stream, op, 100)
 
 
-def timed_region(torch, stream, op, steps, warmup):
+def timed_windows(torch, stream, op, steps, warmup, windows=WINDOWS):
+    """`warmup` untimed launches, then `windows` windows of `steps` launches each, every window between its own pair
+    of events, all back to back on the stream.  Returns the per-launch milliseconds of every window and the wall
+    time of the timed part."""
     for _ in range(warmup):
         op(stream.cuda_stream)
     torch.cuda.synchronize()
     wall0 = time.time()
-    ms = time_launches(torch, stream, op, steps)
-    return ms, time.time() - wall0
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(windows + 1)]
+    ev[0].record(stream)
+    for i in range(windows):
+        for _ in range(steps):
+            op(stream.cuda_stream)
+        ev[i + 1].record(stream)
+    torch.cuda.synchronize()
+    return [ev[i].elapsed_time(ev[i + 1]) / steps for i in range(windows)], time.time() - wall0
+
+
+def spread(ms_list):
+    return {"median": round(statistics.median(ms_list), 6), "min": round(min(ms_list), 6), "max": round(max(ms_list), 6),
+            "windows": len(ms_list)}
 
 
 def roofline(eff_flops, alg_bytes, t, traffic):
@@ -109,14 +133,20 @@ def cpu_baseline(run_all, run_one, eff_flops, sub_flops, what_all, what_one, thr
                       % (what_all, threads, reps, t_sum, t_all, what_one, reps1, t_one, sub_flops / t_one / 1e12)}
 
 
+def timing_note(args):
+    return ("%d warm-up launches, then %d windows of %d back-to-back launches, each between two events on the launch "
+            "stream, operands resident; ms_per_step = median window" % (args.warmup, WINDOWS, args.steps))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=500,
                     help="untimed launches before the timed ones; the shader clock needs about 10 ms of load to settle")
-    ap.add_argument("--config", default="cfg1", help="cfg0 | cfg1 | cfg2 (SpMM; cfg1 is the graded headline) | cfg3 | cfg4 (SpConv2D) | refconv (the "
-                         "reference's own conv test case on its own tensor layout; not graded)")
+    ap.add_argument("--config", default="all",
+                    help="all (default: every graded config, headline cfg1 on top) | cfg0 | cfg1 | cfg2 (SpMM) | cfg3 | cfg4 "
+                         "(SpConv2D) | refconv (the reference's own conv test case on its own tensor layout; not graded)")
     ap.add_argument("--variant", type=int, default=-1, help="force a kernel variant (default: library choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--traffic", default=None,
@@ -135,14 +165,28 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if args.config in P.CONV_CONFIGS:
-        return bench_conv(args, np, torch, S, P)
-    return bench_spmm(args, np, torch, S, P)
+    if args.config != "all":
+        fn = bench_conv if args.config in P.CONV_CONFIGS else bench_spmm
+        print(json.dumps(fn(args, args.config, np, torch, S, P, full=True, cpu=not args.no_cpu)))
+        return
+    # every graded configuration; the CPU leg, the dense GEMM and the cold-cache rotation for the headline only
+    lines = {}
+    for name in ("cfg0", "cfg2", "cfg3", "cfg4", "cfg1"):
+        fn = bench_conv if name in P.CONV_CONFIGS else bench_spmm
+        lines[name] = fn(args, name, np, torch, S, P, full=name == "cfg1", cpu=name == "cfg1" and not args.no_cpu)
+    out = lines["cfg1"]
+    out["configs"] = [{"config": n, "workload": lines[n]["config"]["workload"], "kernel": lines[n]["config"]["kernel"],
+                       "ms_per_step": lines[n]["ms_per_step"], "ms_per_step_spread": lines[n]["ms_per_step_spread"],
+                       "tflops": lines[n]["value"], "pct_mfma_peak": lines[n]["pct_mfma_peak"],
+                       "integer_valued_operands_ms": lines[n]["integer_valued_operands"]["ms_per_step"],
+                       "gate": lines[n]["gate"], "roofline": lines[n]["roofline"]}
+                      for n in ("cfg0", "cfg1", "cfg2", "cfg3", "cfg4")]
+    print(json.dumps(out))
 
 
-def bench_spmm(args, np, torch, S, P):
+def bench_spmm(args, name, np, torch, S, P, full, cpu):
     from oracle import oracle as O  # correctness gate and CPU baseline only
-    c = P.SPMM_CONFIGS[args.config]
+    c = P.SPMM_CONFIGS[name]
     M, K, N, V, d = c["M"], c["K"], c["N"], c["V"], c["d"]
     w = P.make_weight(M, K, V, d, True, 2021, dist=c["a_dist"])
     B = P.make_dense(K, N, 2021, dist=c["b_dist"])
@@ -171,71 +215,30 @@ def bench_spmm(args, np, torch, S, P):
     torch.cuda.synchronize()
     ref_i = O.float_to_half(P.spmm_oracle(wi, Bi))
     if not np.array_equal(dDi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
-        print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
+        print("correctness gate failed (%s): GPU result differs from the CPU oracle" % name, file=sys.stderr)
         sys.exit(1)
 
     ref_loop_ms = reference_loop(torch, stream, op)
-    ms_per_step, wall = timed_region(torch, stream, op, args.steps, args.warmup)
+    windows, wall = timed_windows(torch, stream, op, args.steps, args.warmup)
+    ms_per_step = statistics.median(windows)
     t = ms_per_step * 1e-3
     eff_tflops = eff_flops / t / 1e12
     # the same launch on the integer twin (values of the reference's generator, rand() % 9 - 4): the shader clock
     # under MFMA load depends on the operand values, so this is reported beside the graded figure
-    int_ms, _ = timed_region(torch, stream, opi, args.steps, args.warmup)
+    int_windows, _ = timed_windows(torch, stream, opi, args.steps, args.warmup)
     del mi, dBi, dDi, opi
 
-    # ---- cold-cache variant: rotate operand sets larger than the 256 MB last-level cache
-    nsets = max(2, min(8, int(320e6 // (2 * (K * N + M * N))) + 1))
-    Bs = [dB] + [dB.clone() for _ in range(nsets - 1)]
-    Ds = [dD] + [torch.zeros_like(dD) for _ in range(nsets - 1)]
-    ops = []
-    for i in range(nsets):
-        o = S.SpmmBlockwiseOp(st.variant)
-        o.initialize(mat, N, Bs[i].data_ptr(), Ds[i].data_ptr())
-        ops.append(o)
-    for i in range(nsets):
-        ops[i](stream.cuda_stream)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(args.steps):
-        ops[i % nsets](stream.cuda_stream)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    cold_ms = e0.elapsed_time(e1) / args.steps
-    del Bs, Ds, ops
-
-    # ---- dense fp16 GEMM of the same shape (library GEMM behind torch.matmul) as a reference point
-    Ad = torch.randn((M, K), dtype=torch.float16, device="cuda")
-    for _ in range(5):
-        torch.matmul(Ad, dB, out=dD)
-    torch.cuda.synchronize()
-    e0.record(stream)
-    for _ in range(20):
-        torch.matmul(Ad, dB, out=dD)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    dense_ms = e0.elapsed_time(e1) / 20
-
-    cpu = None
-    if not args.no_cpu:
-        X = M // V
-        XS = max(1, X // 8)
-        sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
-                   values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
-        cpu = cpu_baseline(lambda: P.spmm_oracle(w, B), lambda: P.spmm_oracle(sub, B, nthreads=1), eff_flops,
-                           2.0 * int(w["indptr"][XS]) * V * N, "whole workload (%d panels)" % X,
-                           "the first %d panels" % XS, O.max_threads())
-
-    traffic = measured_traffic(args.config, variant_name) if args.traffic is None else round(float(args.traffic))
+    traffic = measured_traffic(name, variant_name) if args.traffic is None else round(float(args.traffic))
     out = {
-        "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64" if args.config == "cfg1"
-                  else "effective sparse TFLOP/s + %% fp16 MFMA peak, SpMM %s" % args.config,
+        "metric": "effective sparse TFLOP/s + % fp16 MFMA peak, SpMM 4096^3 d=0.1 blk64" if name == "cfg1"
+                  else "effective sparse TFLOP/s + %% fp16 MFMA peak, SpMM %s" % name,
         "value": round(eff_tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6),
+        "ms_per_step_spread": spread(windows),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -243,39 +246,79 @@ def bench_spmm(args, np, torch, S, P):
         "data": "synthetic: seeded Shfl-BW mask + permutation (reference generators, seed 2021), values A %s(%g), B %s(%g)"
                 % (c["a_dist"] + c["b_dist"]),
         "config": {"workload": "%s: Shfl-BW SpMM M=%d K=%d N=%d, block %d, density %g, row-permuted; nnzb=%d"
-                               % (args.config, M, K, N, V, d, nnzb),
-                   "kernel": variant_name, "timing": "events around %d back-to-back launches, operands resident"
-                                                     % args.steps},
+                               % (name, M, K, N, V, d, nnzb),
+                   "kernel": variant_name, "timing": timing_note(args)},
+        "gate": "bit-exact against the CPU oracle on the integer twin",
         "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
         "reference_timing_loop": {"what": "11 warm-ups + 100 launches from an idle GPU (clock still ramping)",
                                   "ms_per_step": round(ref_loop_ms, 6),
                                   "tflops": round(eff_flops / (ref_loop_ms * 1e-3) / 1e12, 1)},
         "integer_valued_operands": {"what": "same mask and shape, values in {-4..4} (the reference's generator)",
-                                    "ms_per_step": round(int_ms, 6),
-                                    "tflops": round(eff_flops / (int_ms * 1e-3) / 1e12, 1)},
+                                    "ms_per_step": round(statistics.median(int_windows), 6),
+                                    "tflops": round(eff_flops / (statistics.median(int_windows) * 1e-3) / 1e12, 1)},
         "dense_equivalent_tflops": round(2.0 * M * N * K / t / 1e12, 1),
         "roofline": roofline(eff_flops, alg_bytes, t, traffic),
-        "cold_cache_ms_per_step": round(cold_ms, 6),
-        "dense_gemm": {"what": "torch.matmul fp16 %dx%dx%d (hipBLASLt/rocBLAS)" % (M, N, K),
-                       "ms": round(dense_ms, 6), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 1)},
-        "cpu_baseline": cpu,
-        "wall_s_timed_region": round(wall, 4),
-        "device": S.device_info(),
     }
-    print(json.dumps(out))
+    if full:
+        # ---- cold-cache variant: rotate operand sets larger than the 256 MB last-level cache
+        nsets = max(2, min(8, int(320e6 // (2 * (K * N + M * N))) + 1))
+        Bs = [dB] + [dB.clone() for _ in range(nsets - 1)]
+        Ds = [dD] + [torch.zeros_like(dD) for _ in range(nsets - 1)]
+        ops = []
+        for i in range(nsets):
+            o = S.SpmmBlockwiseOp(st.variant)
+            o.initialize(mat, N, Bs[i].data_ptr(), Ds[i].data_ptr())
+            ops.append(o)
+        for i in range(nsets):
+            ops[i](stream.cuda_stream)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(args.steps):
+            ops[i % nsets](stream.cuda_stream)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        out["cold_cache_ms_per_step"] = round(e0.elapsed_time(e1) / args.steps, 6)
+        del Bs, Ds, ops
+
+        # ---- dense fp16 GEMM of the same shape (library GEMM behind torch.matmul) as a reference point
+        Ad = torch.randn((M, K), dtype=torch.float16, device="cuda")
+        for _ in range(5):
+            torch.matmul(Ad, dB, out=dD)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(20):
+            torch.matmul(Ad, dB, out=dD)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        dense_ms = e0.elapsed_time(e1) / 20
+        out["dense_gemm"] = {"what": "torch.matmul fp16 %dx%dx%d (hipBLASLt/rocBLAS)" % (M, N, K),
+                             "ms": round(dense_ms, 6), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 1)}
+    out["cpu_baseline"] = None
+    if cpu:
+        X = M // V
+        XS = max(1, X // 8)
+        sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
+                   values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
+        out["cpu_baseline"] = cpu_baseline(lambda: P.spmm_oracle(w, B), lambda: P.spmm_oracle(sub, B, nthreads=1),
+                                           eff_flops, 2.0 * int(w["indptr"][XS]) * V * N,
+                                           "whole workload (%d panels)" % X, "the first %d panels" % XS, O.max_threads())
+    out["wall_s_timed_region"] = round(wall, 4)
+    out["device"] = S.device_info()
+    return out
 
 
-def bench_conv(args, np, torch, S, P):
+def bench_conv(args, name, np, torch, S, P, full, cpu):
     """The sparse Conv2D configs (cfg3, cfg4: NHWC; refconv: the reference's test case on its C-H-W-B / F-H-W-B
     tensors); one step = one exec of the operator, i.e. every launch the chosen form of the convolution puts on
     the stream.  Same JSON shape as the SpMM line."""
     from oracle import oracle as O  # correctness gate and CPU baseline only
-    c = P.CONV_CONFIGS[args.config]
+    c = P.CONV_CONFIGS[name]
     B, H, W, C, F, R, Sx, stride, V, d = [c[k] for k in ("B", "H", "W", "C", "F", "R", "S", "stride", "V", "d")]
     batch_first = c.get("layout") == "chwb"
     if batch_first:
         Ho, Wo = H, W
-        in_shape, out_shape, variant = (C, H, W, B), (F, H, W, B), 4
+        in_shape, out_shape, variant = (C, H, W, B), (F, H, W, B), -1
         oracle = lambda w, x, **kw: P.conv_oracle_batch_first(w, R, Sx, C, x, stride)
     else:
         Ho, Wo = (H + 2 * (R // 2) - R) // stride + 1, (W + 2 * (Sx // 2) - Sx) // stride + 1
@@ -298,9 +341,10 @@ def bench_conv(args, np, torch, S, P):
     opi, fi, dXi, dYi = make_op(wi, xi)
     opi(stream.cuda_stream)
     torch.cuda.synchronize()
+    opi.check()
     ref_i = O.float_to_half(oracle(wi, xi))
     if not np.array_equal(dYi.cpu().numpy().view(np.uint16), ref_i.view(np.uint16)):
-        print("correctness gate failed: GPU result differs from the CPU oracle", file=sys.stderr)
+        print("correctness gate failed (%s): GPU result differs from the CPU oracle" % name, file=sys.stderr)
         sys.exit(1)
 
     w = P.make_weight(F, R * Sx * C, V, d, True, 2021, dist=c["w_dist"])
@@ -311,52 +355,56 @@ def bench_conv(args, np, torch, S, P):
     alg_bytes = nnzb * V * 2 + (nnzb + F // V + 1 + F) * 4 + B * H * W * C * 2 + npix * F * 2
 
     ref_loop_ms = reference_loop(torch, stream, op)
-    ms, wall = timed_region(torch, stream, op, args.steps, args.warmup)
+    windows, wall = timed_windows(torch, stream, op, args.steps, args.warmup)
+    ms = statistics.median(windows)
     t = ms * 1e-3
-    int_ms, _ = timed_region(torch, stream, opi, args.steps, args.warmup)
+    int_windows, _ = timed_windows(torch, stream, opi, args.steps, args.warmup)
+    op.check()
+    opi.check()
     del opi, fi, dXi, dYi
 
-    cpu = None
-    if not args.no_cpu:
+    cpu_line = None
+    if cpu:
         X = F // V
         XS = max(1, X // 8)
         sub = dict(w, nrow=XS * V, indptr=w["indptr"][:XS + 1], indices=w["indices"][:w["indptr"][XS]],
                    values=w["values"][:w["indptr"][XS] * V], row_permute_ids=None)
         # the literal restatement of the reference's loop nest (batch-first layout) runs on one thread
         if batch_first:  # one thread throughout: a bounded sample, the first panels, stands for the workload
-            cpu = cpu_baseline(lambda: oracle(sub, x), lambda: oracle(sub, x), 2.0 * int(w["indptr"][XS]) * V * npix,
-                               2.0 * int(w["indptr"][XS]) * V * npix, "the first %d of %d panels" % (XS, X),
-                               "the same", 1)
+            cpu_line = cpu_baseline(lambda: oracle(sub, x), lambda: oracle(sub, x), 2.0 * int(w["indptr"][XS]) * V * npix,
+                                    2.0 * int(w["indptr"][XS]) * V * npix, "the first %d of %d panels" % (XS, X),
+                                    "the same", 1)
         else:
-            cpu = cpu_baseline(lambda: oracle(w, x),
-                               lambda: oracle(sub, x, nthreads=1), eff_flops,
-                               2.0 * int(w["indptr"][XS]) * V * npix, "whole workload (%d panels)" % X,
-                               "the first %d panels" % XS, O.max_threads())
+            cpu_line = cpu_baseline(lambda: oracle(w, x),
+                                    lambda: oracle(sub, x, nthreads=1), eff_flops,
+                                    2.0 * int(w["indptr"][XS]) * V * npix, "whole workload (%d panels)" % X,
+                                    "the first %d panels" % XS, O.max_threads())
 
     eff_tflops = eff_flops / t / 1e12
     kernel = S.spconv_variant_name(op._state.variant)
-    traffic = measured_traffic(args.config, kernel) if args.traffic is None else round(float(args.traffic))
-    print(json.dumps({
-        "metric": "effective sparse TFLOP/s + %% fp16 MFMA peak, SpConv2D %s" % args.config,
+    traffic = measured_traffic(name, kernel) if args.traffic is None else round(float(args.traffic))
+    return {
+        "metric": "effective sparse TFLOP/s + %% fp16 MFMA peak, SpConv2D %s" % name,
         "value": round(eff_tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 (fp32 accumulate)",
+        "ms_per_step": round(ms, 6), "ms_per_step_spread": spread(windows), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 (fp32 accumulate)",
         "data": "synthetic: seeded Shfl-BW filter mask + permutation (seed 2021), filter %s(%g), input %s(%g)"
                 % (c["w_dist"] + c["x_dist"]),
         "config": {"workload": "%s: sparse Conv2D %s %dx%dx%dx%d -> %d, %dx%d stride %d, block %d, density %g; "
-                               "nnzb=%d" % (args.config, "C-H-W-B / F-H-W-B, B x H x W x C =" if batch_first else "NHWC",
+                               "nnzb=%d" % (name, "C-H-W-B / F-H-W-B, B x H x W x C =" if batch_first else "NHWC",
                                             B, H, W, C, F, R, Sx, stride, V, d, nnzb),
-                   "kernel": kernel, "timing": "events around %d back-to-back execs, operands resident" % args.steps},
+                   "kernel": kernel, "timing": timing_note(args)},
+        "gate": "bit-exact against the CPU oracle on the integer twin",
         "pct_mfma_peak": round(100.0 * eff_tflops / MFMA_F16_PEAK_TFLOPS, 2),
         "reference_timing_loop": {"what": "11 warm-ups + 100 execs from an idle GPU (clock still ramping)",
                                   "ms_per_step": round(ref_loop_ms, 6),
                                   "tflops": round(eff_flops / (ref_loop_ms * 1e-3) / 1e12, 1)},
         "integer_valued_operands": {"what": "same mask and shape, values in {-4..4} (the reference's generator)",
-                                    "ms_per_step": round(int_ms, 6),
-                                    "tflops": round(eff_flops / (int_ms * 1e-3) / 1e12, 1)},
+                                    "ms_per_step": round(statistics.median(int_windows), 6),
+                                    "tflops": round(eff_flops / (statistics.median(int_windows) * 1e-3) / 1e12, 1)},
         "dense_equivalent_tflops": round(2.0 * npix * F * R * Sx * C / t / 1e12, 1),
-        "roofline": roofline(eff_flops, alg_bytes, t, traffic), "cpu_baseline": cpu,
-        "wall_s_timed_region": round(wall, 4), "device": S.device_info()}))
+        "roofline": roofline(eff_flops, alg_bytes, t, traffic), "cpu_baseline": cpu_line,
+        "wall_s_timed_region": round(wall, 4), "device": S.device_info()}
 
 
 if __name__ == "__main__":

@@ -192,21 +192,28 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  *   H, W are the INPUT extents; padding is R/2, S/2 ("same" for stride 1, as the
  *   reference's col2im, spconv/conv_format.h:77-81); Ho = (H + 2*(R/2) - R)/stride + 1.
  * Preconditions: filter synced, bcol == 1, C % 8 == 0, F % 8 == 0.
- * init allocates device scratch inside the filter object (freed with it; states made from one
- * filter with equal scratch size share it, so launch them on one stream); exec only launches, in
- * order on `stream`: a layout pass over the input, the SpMM kernel, and the transpose to NHWC.
- * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice, 5 when B % 8 == 0, else 0):
- *   variant 0 = plane form: the input is rewritten once per call as channel-major padded
+ * init allocates device scratch inside the filter object (freed with it or by shflbw_weight_release_scratch):
+ * the gather ids once per (form, B, H, W, stride), and per (form, geometry, IFMap, OFMap) the buffers the launches
+ * write - states over different tensors never share those and may run on different streams.  At most
+ * SHFLBW_CONV_SCRATCH_DEPTH such buffers exist per filter: initialising a state over one more tensor pair recycles
+ * the buffers of the least recently initialised one (no allocation, no copy when the geometry is the same), whose
+ * state must not be executed afterwards.  exec only launches, in order on `stream`.
+ * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice):
+ *   variant 0 = plane form, three launches: the input is rewritten once per call as channel-major padded
  *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
  *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,
- *     its address generation is the per-id offset of the gather;
- *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads);
- *   variant 2 = explicit im2col matrix, SpMM, transpose;
- *   variant 3 = the steps of variant 0 in one persistent launch;
- *   variant 5 = plane form with the batch innermost in the planes and in the filter-major result (B % 8 == 0):
+ *     its address generation is the per-id offset of the gather; a tile transpose writes NHWC;
+ *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads; block sizes 32, 64, 128);
+ *   variant 2 = plane form with the batch innermost in the planes and in the filter-major result (B % 8 == 0):
  *     every tap offset is then a multiple of 16 bytes, one copy of the planes serves all taps, and the result
- *     holds output pixels only.
+ *     holds output pixels only; three launches;
+ *   variant 3 = the steps of variant 2 in ONE persistent launch (B % 8 == 0): every XCD of the GPU rewrites the
+ *     input, runs the SpMM and writes NHWC for its own range of output columns, in its own L2; the phases are
+ *     counted between the workgroups of an XCD.  Needs a device that deals consecutive workgroups to consecutive
+ *     XCDs (checked at init; SHFLBW_ERR_UNSUPPORTED otherwise).  Its waits are bounded: should one run out the launch still ends,
+ *     and shflbw_spconv_check reports it.
  * ------------------------------------------------------------------------- */
+#define SHFLBW_CONV_SCRATCH_DEPTH 4
 typedef struct shflbw_spconv_state {
     size_t shared_mem_size;
     unsigned grid_dim[3];
@@ -231,19 +238,20 @@ typedef struct shflbw_spconv_state {
     /* Device scratch owned by the filter and the state of the SpMM launch in the middle.
      * Plane form (variant 0): `planes` holds the input as channel-major zero-padded planes
      * [plane_copies][stride*stride][C][plane_pitch]; a "pixel" of the GEMM is a position
-     * b*plane_rows*plane_cols + i*plane_cols + j of that padded grid, np = B*plane_rows*plane_cols of
-     * them, and result_fm is [F][np].  im2col form (variant 2): im2col is the matrix [R*S*C][np],
-     * np = B*Ho*Wo rounded up to 64, result_fm [F][np].  Batch-innermost forms (variants 4, 5): `planes` is
+     * b*plane_rows*plane_cols + i*plane_cols + j of that padded grid, np = ncols = B*plane_rows*plane_cols of
+     * them, and result_fm is [F][np].  Batch-innermost forms (variants 2, 4): `planes` is
      * [stride*stride][C][plane_pitch] with position (i*plane_cols + j)*B + b, plane_rows = Ho + (R-1)/stride,
-     * plane_cols = Wo + (S-1)/stride; ncols = Ho*plane_cols*B columns of the GEMM; result_fm (variant 5) is
-     * [F][Ho*Wo*B]. */
-    void* im2col;
+     * plane_cols = Wo + (S-1)/stride; ncols = Ho*plane_cols*B columns of the GEMM; result_fm (variant 2) is
+     * [F][Ho*Wo*B].  Fused form (variant 3): the columns are those of variant 2, cols_per_xcd of them per XCD;
+     * `planes` holds xcds slabs [stride*stride*C + 1][plane_pitch] (the positions one XCD's columns read),
+     * result_fm xcds results [F][cols_per_xcd], `sync` the counters (all zero between launches). */
     void* result_fm;
     int np;
     void* planes;
     int plane_rows, plane_cols, plane_pitch, plane_copies;
-    int ncols;  /* fused form: columns of the GEMM = plane positions of output rows, B*Ho*plane_cols; result_fm is [F][ncols] */
-    void* sync; /* fused form: synchronisation words in the scratch, all zero between launches */
+    int ncols;
+    int xcds, cols_per_xcd;
+    void* sync;
     shflbw_spmm_state spmm;
 } shflbw_spconv_state;
 
@@ -273,6 +281,12 @@ int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* fil
 int shflbw_spconv_exec_static(const shflbw_weight* filter, int B, int H, int W, int stride,
                               const void* IFMap, void* OFMap, void* stream);
 
+/* No counterpart in the reference.  Synchronous: waits for the device, then tells whether every launch of the
+ * fused form (variant 3) on this state's scratch ran to completion: SHFLBW_ERR_HIP when the workgroups were not dealt to
+ * the XCDs the way init had checked, or when a bounded wait between its phases ran out (the output of that launch
+ * is then invalid; the scratch is reset for further launches).  SHFLBW_OK for every other form. */
+int shflbw_spconv_check(const shflbw_spconv_state* state);
+
 /* Forms of the convolution shflbw_spconv_init_variant accepts, and a short name for each. */
 int shflbw_spconv_variant_count(void);
 const char* shflbw_spconv_variant_name(int variant);
@@ -280,6 +294,8 @@ const char* shflbw_spconv_variant_name(int variant);
  * dangle (the reference has no scratch; its states dangle the same way when the filter is
  * re-initialised, spmm/blockwise_op.h:118-122). */
 int shflbw_weight_release_scratch(shflbw_weight* filter);
+/* Device bytes and number of buffers of convolution scratch the filter holds at the moment. */
+int shflbw_weight_scratch_bytes(const shflbw_weight* filter, size_t* bytes, int* buffers);
 
 /* sizeof the two state structs as this library was compiled, for FFI mirrors to check their layout. */
 void shflbw_abi_sizes(size_t* spmm_state_bytes, size_t* spconv_state_bytes);

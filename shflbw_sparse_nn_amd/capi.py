@@ -25,6 +25,7 @@ EXPORTS = [
     "shflbw_spconv_init", "shflbw_spconv_init_variant", "shflbw_spconv_exec",
     "shflbw_spconv_exec_static", "shflbw_spconv_init_chwb", "shflbw_spconv_host_reference_chwb",
     "shflbw_spconv_variant_count", "shflbw_spconv_variant_name", "shflbw_weight_release_scratch",
+    "shflbw_spconv_check", "shflbw_weight_scratch_bytes",
     "shflbw_spmm_host_reference", "shflbw_spconv_host_reference",
     "shflbw_abi_sizes", "shflbw_device_info",
 ]
@@ -72,9 +73,10 @@ class SpconvState(C.Structure):
                 ("init_success", C.c_int), ("variant", C.c_int), ("args", _SpconvArgs),
                 ("Ho", C.c_int), ("Wo", C.c_int),
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("panel_ptr", C.c_void_p),
-                ("brow", C.c_int), ("im2col", C.c_void_p), ("result_fm", C.c_void_p), ("np", C.c_int),
+                ("brow", C.c_int), ("result_fm", C.c_void_p), ("np", C.c_int),
                 ("planes", C.c_void_p), ("plane_rows", C.c_int), ("plane_cols", C.c_int), ("plane_pitch", C.c_int),
-                ("plane_copies", C.c_int), ("ncols", C.c_int), ("sync", C.c_void_p), ("spmm", SpmmState)]
+                ("plane_copies", C.c_int), ("ncols", C.c_int), ("xcds", C.c_int), ("cols_per_xcd", C.c_int),
+                ("sync", C.c_void_p), ("spmm", SpmmState)]
 
 
 _lib = None
@@ -129,6 +131,8 @@ def load():
     lib.shflbw_spconv_variant_name.restype = C.c_char_p
     lib.shflbw_spconv_variant_name.argtypes = [ci]
     lib.shflbw_weight_release_scratch.argtypes = [vp]
+    lib.shflbw_spconv_check.argtypes = [C.POINTER(SpconvState)]
+    lib.shflbw_weight_scratch_bytes.argtypes = [vp, C.POINTER(sz), ip]
     lib.shflbw_spmm_host_reference.argtypes = [vp, ci, vp, cf, vp, cf, vp]
     lib.shflbw_spconv_host_reference.argtypes = [vp, ci, ci, ci, ci, vp, vp]
     lib.shflbw_abi_sizes.restype = None

@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "shflbw.h"
@@ -27,6 +28,8 @@ namespace shflbw {
         }                                                                                               \
     } while (0)
 
+static void release_conv_scratch(shflbw_weight* w);
+
 void clear_device(shflbw_weight* w)
 {
     void** bufs[] = {&w->d_meta, &w->d_values, &w->d_group_ptr, &w->d_packed_indices, &w->d_packed_indices_pm,
@@ -35,9 +38,18 @@ void clear_device(shflbw_weight* w)
         if (*b) (void)hipFree(*b);
         *b = nullptr;
     }
-    for (auto& sc : w->conv_scratch)
-        if (sc.ptr) (void)hipFree(sc.ptr);
-    w->conv_scratch.clear();
+    release_conv_scratch(w);
+}
+
+// frees every device buffer the convolution inits of this weight allocated (the caller holds scratch_lock or owns w)
+void release_conv_scratch(shflbw_weight* w)
+{
+    for (auto& e : w->conv_ids)
+        if (e.ptr) (void)hipFree(e.ptr);
+    for (auto& e : w->conv_bulk)
+        if (e.ptr) (void)hipFree(e.ptr);
+    w->conv_ids.clear();
+    w->conv_bulk.clear();
 }
 
 static int upload_one(void** dst, const void* src, size_t bytes)
@@ -65,19 +77,19 @@ int upload(shflbw_weight* w)
     return SHFLBW_OK;
 }
 
-// compute units of the current device, looked up once per process
+// compute units of the current device, looked up once per device
 static int device_compute_units()
 {
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cached = n;
-        else
-            cached = 256;
+    static std::mutex lock;
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    std::lock_guard<std::mutex> guard(lock);
+    if (cached[dev] == 0) {
+        int n = 0;
+        cached[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
     }
-    return cached;
+    return cached[dev];
 }
 
 static const SpmmVariant* find_spmm_variant(int brow, int variant, int* n_for_brow)
@@ -128,12 +140,12 @@ static bool spmm_variant_offsets32(const SpmmVariant* v) { return v && v->name[0
 //    at the same time and share it in their L2 (16 tiles: 15 % slower).
 // Inside these bounds: equal to 28 % faster (M = 4096, K = 1024, N = 4096, density 0.2: 15.1 against 16.5 us;
 // M = 8192, density 0.3: 31.3 against 38.7 us).
-static int auto_spmm_variant(const shflbw_weight* w, int N)
+static int auto_spmm_variant(const shflbw_weight* w, int N, bool allow_slab)
 {
     const int brow = w->brow, X = w->nrow / w->brow;
     int count = 0;
     const SpmmVariant* all = spmm_variants(&count);
-    if (brow == 32 && !w->packed_slab.empty() && w->ncol >= 384 && X > 0) {
+    if (allow_slab && brow == 32 && !w->packed_slab.empty() && w->ncol >= 384 && X > 0) {
         int seen = 0;
         for (int i = 0; i < count; i++) {
             if (all[i].V != brow) continue;
@@ -170,10 +182,9 @@ struct PlaneForm {
     long pitch;     // values per channel row of the plane tensor
     long rows;      // channel rows: copies * stride^2 * C
     size_t slots;   // padded kept-vector slots of the filter
-    long ncols;     // columns of the fused form: plane positions of output rows only, B * Ho * PW
     int Ho, Wo;
-    size_t planes_bytes, dm_bytes, ids_bytes, sync_bytes; // scratch = planes | result_fm | ids | ids_pm | sync words
-    size_t total_bytes() const { return planes_bytes + dm_bytes + 2 * ids_bytes + sync_bytes; }
+    size_t planes_bytes, dm_bytes, ids_bytes; // planes | result_fm, and (the entry point without allocation) | ids | ids_pm behind them
+    size_t total_bytes() const { return planes_bytes + dm_bytes + 2 * ids_bytes; }
 };
 
 static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int stride, PlaneForm* g)
@@ -201,8 +212,6 @@ static int plane_form_geometry(const shflbw_weight* f, int B, int H, int W, int 
     g->ids_bytes = up256(g->slots * sizeof(int) + 64);
     g->Ho = (H + 2 * ph - f->R) / s + 1;
     g->Wo = (W + 2 * pw - f->S) / s + 1;
-    g->ncols = (long)B * g->Ho * g->PW;
-    g->sync_bytes = (size_t)conv_sync_lines((int)((g->ncols + 255) / 256)) * SYNC_LINE * sizeof(int); // column tiles are 256 wide at least
     return SHFLBW_OK;
 }
 
@@ -230,10 +239,8 @@ static void fill_spmm_launch_args(const shflbw_spmm_state* state, int BN, SpmmLa
     a.alpha = state->args.alpha;
     a.beta = state->args.beta;
     a.num_cus = device_compute_units();
-    a.img_cols = 1, a.img_skip = 0;
     a.ldd = a.N;
     a.dmap_row = a.dmap_valid = 0, a.dmap_magic = 0;
-    a.tile_arrivals = nullptr;
     // rows of B one column tile can touch: above about 2.5 MB they do not stay in the 4 MB L2 of an XCD
     // from one round of tiles to the next, and alternating the direction of the walk pays (measured:
     // +1 % at 2 MB, -4 % at 3 MB, -7 % at 4 MB, -13 % at 8 MB)
@@ -259,8 +266,11 @@ const char* shflbw_spmm_variant_name(int brow, int variant)
     return v ? v->name : "";
 }
 
-int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C,
-                             void* D, float alpha, float beta, int variant)
+// `gather_only`: the caller will point the gather at something other than a K x N matrix (the planes of a
+// convolution, ids rewritten as element offsets), which only the variants that gather rows by id can walk: the
+// variants that hold all K rows of B in LDS are left out of the automatic choice and refused when forced.
+static int spmm_init_impl(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C, void* D,
+                          float alpha, float beta, int variant, bool gather_only)
 {
     if (!state) return SHFLBW_ERR_INVALID;
     memset(state, 0, sizeof(*state));
@@ -292,7 +302,7 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     // the role-split kernels address the rows of B with 32-bit byte offsets
     const bool wide_b = (unsigned long long)w->ncol * (unsigned long long)N * 2ull + (unsigned long long)N * 2ull > 0xffffffffull;
     if (variant < 0) {
-        variant = auto_spmm_variant(w, N);
+        variant = auto_spmm_variant(w, N, !gather_only);
         if (wide_b) { // first variant of this block size with 64-bit addressing
             int n = 0;
             find_spmm_variant(w->brow, 0, &n);
@@ -306,6 +316,10 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     const SpmmVariant* v = find_spmm_variant(w->brow, variant, nullptr);
     if (!v) {
         set_error("spmm_init: no tile variant %d for block size %d", variant, w->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (v->max_k > 0 && gather_only) {
+        set_error("spmm_init: tile variant %s holds the rows of B in LDS and cannot walk the planes of a convolution", v->name);
         return SHFLBW_ERR_UNSUPPORTED;
     }
     if (v->max_k > 0 && (w->ncol > v->max_k || w->packed_slab.empty())) {
@@ -355,6 +369,12 @@ int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, i
     return SHFLBW_OK;
 }
 
+int shflbw_spmm_init_variant(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C,
+                             void* D, float alpha, float beta, int variant)
+{
+    return spmm_init_impl(state, w, N, B, C, D, alpha, beta, variant, false);
+}
+
 int shflbw_spmm_init(shflbw_spmm_state* state, const shflbw_weight* w, int N, const void* B, const void* C, void* D,
                      float alpha, float beta)
 {
@@ -387,9 +407,16 @@ int shflbw_spconv_init(shflbw_spconv_state* state, const shflbw_weight* f, int B
     return shflbw_spconv_init_variant(state, f, B, H, W, stride, IFMap, OFMap, -1);
 }
 
+} // extern "C"
+
+namespace {
+
+// forms of the convolution (shflbw_spconv_variant_name)
+enum ConvForm { FORM_PLANES = 0, FORM_DIRECT = 1, FORM_BPLANES = 2, FORM_FUSED = 3, FORM_CHWB = 4, FORM_COUNT = 5 };
+
 // Argument checks of a convolution and every field of the state that does not depend on device scratch.
-static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                             const void* IFMap, void* OFMap, int variant)
+int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                      const void* IFMap, void* OFMap, int variant)
 {
     if (!state) return SHFLBW_ERR_INVALID;
     memset(state, 0, sizeof(*state));
@@ -413,7 +440,7 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
         set_error("spconv_init: non-positive B, H, W or stride");
         return SHFLBW_ERR_INVALID;
     }
-    if (variant != 4 && ((f->C % 8) != 0 || (f->F % 8) != 0)) { // NHWC forms move 8 channels / 8 filters at a time
+    if (variant != FORM_CHWB && ((f->C % 8) != 0 || (f->F % 8) != 0)) { // NHWC forms move 8 channels / 8 filters at a time
         set_error("spconv_init: C and F must be multiples of 8 (got %d, %d)", f->C, f->F);
         return SHFLBW_ERR_SHAPE;
     }
@@ -427,14 +454,16 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
         set_error("spconv_init: empty output (%d x %d)", Ho, Wo);
         return SHFLBW_ERR_SHAPE;
     }
-    if (variant < 0 || variant >= shflbw_spconv_variant_count()) {
-        set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = im2col form, 3 = plane form fused into one launch)", variant);
+    if (variant < 0 || variant >= FORM_COUNT) {
+        set_error("spconv_init: variant %d does not exist (0 = plane form, 1 = direct kernel, 2 = batch-innermost plane "
+                  "form, 3 = batch-innermost plane form fused into one launch)", variant);
         return SHFLBW_ERR_INVALID;
     }
-    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
-    if (variant == 1) {
+    if (variant == FORM_DIRECT) {
+        const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
         if (!v) {
-            set_error("spconv_init: no direct kernel for block size %d", f->brow);
+            set_error("spconv_init: the direct kernel (variant 1) exists for block sizes 32, 64 and 128, not %d; "
+                      "the plane forms (0, 2, 3) serve every block size", f->brow);
             return SHFLBW_ERR_UNSUPPORTED;
         }
         if ((unsigned long long)B * H * W * f->C > 0x7fffffffull) {
@@ -471,181 +500,240 @@ static int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f,
     return SHFLBW_OK;
 }
 
-// Points a state of the plane form at its scratch (planes | result_fm | ids | ids_pm, laid out by `g`) and sets
-// up the SpMM launch in the middle.  The ids must be in the scratch when the state is executed.
-static int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, const PlaneForm& g, char* scratch,
-                           bool fused)
+size_t up256(size_t n) { return (n + 255) / 256 * 256; }
+
+// The gather ids of one (form, geometry) on the device: `ids_bytes` of slot-ordered ids, then the same ids in the
+// producer-major order of every 64-slot group.  `offset_of(k)` maps a kept column k = (r*S + t)*C + c to its element
+// offset in the layout-transformed input; padding slots (k < 0) get `zero_id`, the offset of a row of zeros.  Built
+// and uploaded on the first call for a key, found afterwards.  The caller holds the weight's scratch_lock.
+template <class OffsetOf>
+int conv_ids_for(shflbw_weight* fw, const int (&key)[5], int zero_id, OffsetOf offset_of, const int** ids, const int** ids_pm)
 {
-    state->planes = scratch;
-    state->result_fm = scratch + g.planes_bytes;
+    const size_t slots = fw->packed_indices.size();
+    const size_t ids_bytes = up256(slots * sizeof(int) + 64);
+    for (auto& e : fw->conv_ids)
+        if (memcmp(e.key, key, sizeof(key)) == 0 && e.bytes == 2 * ids_bytes) {
+            *ids = (const int*)e.ptr;
+            *ids_pm = (const int*)((const char*)e.ptr + ids_bytes);
+            return SHFLBW_OK;
+        }
+    std::vector<int> h(2 * ids_bytes / sizeof(int), 0);
+    int* pm = h.data() + ids_bytes / sizeof(int);
+    for (size_t q = 0; q < slots; q++) {
+        const int k = fw->packed_indices[q];
+        const int id = k < 0 ? zero_id : offset_of(k);
+        h[q] = id;
+        const size_t grp = q / 64; // producer-major order inside every 64-slot group
+        const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
+        pm[grp * 64 + 16 * p + 4 * j + r] = id;
+    }
+    void* d = nullptr;
+    SHFLBW_HIP_TRY(hipMalloc(&d, 2 * ids_bytes));
+    if (hipMemcpy(d, h.data(), 2 * ids_bytes, hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipFree(d);
+        set_error("spconv_init: cannot upload the gather ids");
+        return SHFLBW_ERR_HIP;
+    }
+    fw->conv_ids.push_back(shflbw_weight::ConvIds{{key[0], key[1], key[2], key[3], key[4]}, d, 2 * ids_bytes});
+    *ids = (const int*)d;
+    *ids_pm = (const int*)((const char*)d + ids_bytes);
+    return SHFLBW_OK;
+}
+
+// The bulk scratch (layout-transformed input, filter-major result, counters) of a state: the buffer of an equal
+// (form, geometry, tensors) if there is one; else a new one, cleared, while fewer than CONV_BULK_DEPTH exist; else the
+// least recently handed out one - as it is when it served the same geometry (what has to be zero in it still is: the
+// parts of the planes no launch writes, the counters every launch leaves at zero), freed and allocated anew
+// otherwise.  The caller holds the weight's scratch_lock.
+int conv_bulk_for(shflbw_weight* fw, const int (&key)[5], const void* in, const void* out, size_t bytes, char** ptr)
+{
+    auto& pool = fw->conv_bulk;
+    fw->bulk_clock++;
+    for (auto& e : pool)
+        if (e.bytes == bytes && memcmp(e.key, key, sizeof(key)) == 0 && e.in == in && e.out == out) {
+            e.stamp = fw->bulk_clock;
+            *ptr = (char*)e.ptr;
+            return SHFLBW_OK;
+        }
+    if ((int)pool.size() >= shflbw_weight::CONV_BULK_DEPTH) {
+        size_t lru = 0;
+        for (size_t i = 1; i < pool.size(); i++)
+            if (pool[i].stamp < pool[lru].stamp) lru = i;
+        if (pool[lru].bytes == bytes && memcmp(pool[lru].key, key, sizeof(key)) == 0) {
+            pool[lru].in = in, pool[lru].out = out, pool[lru].stamp = fw->bulk_clock;
+            *ptr = (char*)pool[lru].ptr;
+            return SHFLBW_OK;
+        }
+        (void)hipFree(pool[lru].ptr);
+        pool.erase(pool.begin() + lru);
+    }
+    void* d = nullptr;
+    if (hipMalloc(&d, bytes) != hipSuccess) {
+        set_error("spconv_init: cannot allocate %zu bytes of device scratch", bytes);
+        return SHFLBW_ERR_HIP;
+    }
+    // cleared before any stream can launch on it (the caller's stream need not be ordered behind the one the clear runs on)
+    if (hipMemset(d, 0, bytes) != hipSuccess || hipStreamSynchronize(nullptr) != hipSuccess) {
+        (void)hipFree(d);
+        set_error("spconv_init: cannot clear %zu bytes of device scratch", bytes);
+        return SHFLBW_ERR_HIP;
+    }
+    pool.push_back(shflbw_weight::ConvBulk{{key[0], key[1], key[2], key[3], key[4]}, in, out, d, bytes, fw->bulk_clock});
+    *ptr = (char*)d;
+    return SHFLBW_OK;
+}
+
+// Sets up the SpMM launch in the middle of a plane form: N columns, the planes as B, `result` as D, the rewritten ids
+// (element offsets: one id apart is one value apart) and `id_space` as the extent the ids address.
+int bind_middle(shflbw_spconv_state* state, const shflbw_weight* f, long N, const void* planes, void* result,
+                const int* ids, const int* ids_pm, long id_space)
+{
+    // only the variants that gather rows by id can walk the planes; the first one of the block size (role-split)
+    int rc = spmm_init_impl(&state->spmm, f, (int)N, planes, nullptr, result, 1.f, 0.f, -1, true);
+    if (rc != SHFLBW_OK) return rc;
+    state->spmm.packed_indices = ids;
+    state->spmm.packed_indices_pm = ids_pm;
+    state->spmm.ldb_bytes = 2;
+    state->spmm.args.K = (int)id_space;
+    return SHFLBW_OK;
+}
+
+void copy_middle_launch_figures(shflbw_spconv_state* state)
+{
+    state->shared_mem_size = state->spmm.shared_mem_size;
+    state->grid_dim[0] = state->spmm.grid_dim[0];
+    state->block_dim[0] = state->spmm.block_dim[0];
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[1] = state->block_dim[2] = 1;
+}
+
+// Form 0.  Points a state at its scratch (laid out by `g`) and sets up the SpMM launch in the middle.
+int bind_plane_form(shflbw_spconv_state* state, const shflbw_weight* f, const PlaneForm& g, char* planes, char* result,
+                    const int* ids, const int* ids_pm)
+{
+    state->planes = planes;
+    state->result_fm = result;
     state->np = (int)g.np;
     state->plane_rows = g.PH;
     state->plane_cols = g.PW;
     state->plane_pitch = (int)g.pitch;
     state->plane_copies = g.copies;
-    state->ncols = (int)g.ncols;
-    state->sync = scratch + g.planes_bytes + g.dm_bytes + 2 * g.ids_bytes;
-    // the three-launch form computes every plane position, the fused form only those of output rows
-    int rc = fused ? shflbw_spmm_init_variant(&state->spmm, f, (int)g.ncols, state->planes, nullptr, state->result_fm, 1.f, 0.f, 0)
-                   : shflbw_spmm_init(&state->spmm, f, (int)g.np, state->planes, nullptr, state->result_fm, 1.f, 0.f);
+    state->ncols = (int)g.np;
+    int rc = bind_middle(state, f, g.np, planes, result, ids, ids_pm, (g.rows + 1) * g.pitch);
     if (rc != SHFLBW_OK) return rc;
-    if (fused) {
-        const ConvFusedKernel* k = conv_fused_kernel(f->brow);
-        if (!k) {
-            set_error("spconv_init: no fused kernel for block size %d", f->brow);
-            return SHFLBW_ERR_UNSUPPORTED;
-        }
-        SHFLBW_HIP_TRY(k->prepare());
-        state->spmm.shared_mem_size = (size_t)k->lds_bytes;
-        state->spmm.grid_dim[0] = (unsigned)((f->nrow / f->brow) * ((g.ncols + k->BN - 1) / k->BN));
-        state->spmm.block_dim[0] = (unsigned)k->threads;
-    }
-    // the gather walks the planes: ids are element offsets, one id apart is one value apart
-    state->spmm.packed_indices = (const int*)(scratch + g.planes_bytes + g.dm_bytes);
-    state->spmm.packed_indices_pm = (const int*)(scratch + g.planes_bytes + g.dm_bytes + g.ids_bytes);
-    state->spmm.ldb_bytes = 2;
-    state->spmm.args.K = (int)((g.rows + 1) * g.pitch); // extent of the id space
-    state->shared_mem_size = state->spmm.shared_mem_size; // the figures of the middle (SpMM) launch
-    state->grid_dim[0] = state->spmm.grid_dim[0];
-    state->block_dim[0] = state->spmm.block_dim[0];
-    state->grid_dim[1] = state->grid_dim[2] = 1;
-    state->block_dim[1] = state->block_dim[2] = 1;
+    copy_middle_launch_figures(state);
     state->init_success = 1;
     return SHFLBW_OK;
 }
 
-static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                             const void* IFMap, void* OFMap, int variant);
-
-int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                               const void* IFMap, void* OFMap, int variant)
+int init_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride, const void* IFMap,
+                void* OFMap)
 {
-    if (variant == 4) {
-        if (state) memset(state, 0, sizeof(*state));
-        set_error("spconv_init: form 4 works on C-H-W-B / F-H-W-B tensors; call shflbw_spconv_init_chwb");
-        return SHFLBW_ERR_INVALID;
-    }
-    // the library's choice: the batch-innermost plane form where the batch allows it (one copy of the planes instead
-    // of two, no dead plane rows in the result: cfg3 22.9 against 25.3 us, cfg4 24.0 against 25.9), else the plane form
-    if (variant < 0) variant = B > 0 && B % 8 == 0 ? 5 : 0;
-    if (variant == 5) return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, 5);
-    int frc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
-    if (frc != SHFLBW_OK) return frc;
-    const int Ho = state->Ho, Wo = state->Wo;
-    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr); // the direct kernel, where one exists
-    const long npix = (long)B * Ho * Wo;
+    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, FORM_PLANES);
+    if (rc != SHFLBW_OK) return rc;
+    PlaneForm g;
+    if ((rc = plane_form_geometry(f, B, H, W, stride, &g)) != SHFLBW_OK) return rc;
     // The scratch cache is bookkeeping of the handle, not part of the weight's value; it is the one member an
     // init call changes, under its lock.
     shflbw_weight* fw = const_cast<shflbw_weight*>(f);
     std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
-    const int key[5] = {variant, B, H, W, stride};
-    auto cached_scratch = [&](size_t bytes, bool* fresh) -> void* {
-        for (auto& sc : fw->conv_scratch)
-            if (sc.bytes == bytes && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap) {
-                *fresh = false;
-                return sc.ptr;
-            }
-        void* ptr = nullptr;
-        if (hipMalloc(&ptr, bytes) != hipSuccess) return nullptr;
-        shflbw_weight::Scratch sc{bytes, ptr, {key[0], key[1], key[2], key[3], key[4]}, IFMap, OFMap};
-        fw->conv_scratch.push_back(sc);
-        *fresh = true;
-        return ptr;
-    };
-    if (variant == 0 || variant == 3) {
-        // plane forms: geometry of the phase planes (see spconv_gfx950.hip)
-        PlaneForm g;
-        int grc = plane_form_geometry(f, B, H, W, stride, &g);
-        if (grc != SHFLBW_OK) return grc;
-        const int s = stride;
-        const long PW = g.PW, pitch = g.pitch;
-        const int copies = g.copies;
-        const size_t slots = g.slots, planes_bytes = g.planes_bytes, dm_bytes = g.dm_bytes, ids_bytes = g.ids_bytes;
-        bool fresh = false;
-        char* scratch = (char*)cached_scratch(g.total_bytes(), &fresh);
-        if (!scratch) {
-            set_error("spconv_init: cannot allocate %zu bytes of device scratch", g.total_bytes());
-            return SHFLBW_ERR_HIP;
-        }
-        int* d_ids = (int*)(scratch + planes_bytes + dm_bytes);
-        int* d_ids_pm = (int*)(scratch + planes_bytes + dm_bytes + ids_bytes);
-        if (fresh) {
-            // the tail of every channel row and the positions no image covers are read (for results
-            // nobody uses) but never written
-            SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes));
-            // the synchronisation words of the fused form start at zero (every launch leaves them so)
-            SHFLBW_HIP_TRY(hipMemset(scratch + planes_bytes + dm_bytes + 2 * ids_bytes, 0, g.sync_bytes));
-            // kept-column id k = (r*S + t)*C + c  ->  element offset of (copy, phase, channel) row + tap offset
-            std::vector<int> ids(slots), ids_pm(slots);
-            for (size_t q = 0; q < slots; q++) {
-                const int k = f->packed_indices[q];
-                if (k < 0) { // padding slot: the row of zeros behind the last channel row
-                    ids[q] = (int)(g.rows * pitch);
-                    continue;
-                }
-                const int c = k % f->C, tap = k / f->C, r = tap / f->S, t = tap % f->S;
-                const long shift = (long)(r / s) * PW + t / s;
-                const int copy = copies == 2 ? (int)(shift & 1) : 0;
-                const int phase = (r % s) * s + t % s;
-                ids[q] = (int)((((long)copy * s * s + phase) * f->C + c) * pitch + shift - copy);
-            }
-            for (size_t q = 0; q < slots; q++) { // producer-major order inside every 64-slot group
-                const size_t grp = q / 64;
-                const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
-                ids_pm[grp * 64 + 16 * p + 4 * j + r] = ids[q];
-            }
-            SHFLBW_HIP_TRY(hipMemcpy(d_ids, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
-            SHFLBW_HIP_TRY(hipMemcpy(d_ids_pm, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
-        }
-        return bind_plane_form(state, f, g, scratch, variant == 3);
-    }
-    if (variant == 2) {
-        // im2col form: scratch for the im2col matrix [K][np] and the filter-major result [F][np]
-        const long np = (npix + 63) / 64 * 64;
-        const long K = (long)f->R * f->S * f->C;
-        if (np > 0x7fffffffL || (unsigned long long)K * (unsigned long long)np * 2ull > 0xffffffffull) {
-            set_error("spconv_init: problem too large for the im2col form (im2col matrix of %ld x %ld)", K, np);
-            return SHFLBW_ERR_UNSUPPORTED;
-        }
-        const size_t bm_bytes = (size_t)K * np * 2, dm_bytes = (size_t)f->F * np * 2;
-        bool fresh = false;
-        void* scratch = cached_scratch(bm_bytes + dm_bytes, &fresh);
-        if (!scratch) {
-            set_error("spconv_init: cannot allocate %zu bytes of device scratch", bm_bytes + dm_bytes);
-            return SHFLBW_ERR_HIP;
-        }
-        state->im2col = scratch;
-        state->result_fm = (char*)scratch + bm_bytes;
-        state->np = (int)np;
-        int rc = shflbw_spmm_init(&state->spmm, f, (int)np, state->im2col, nullptr, state->result_fm, 1.f, 0.f);
-        if (rc != SHFLBW_OK) return rc;
-    }
-    if (variant == 1) {
-        state->shared_mem_size = (size_t)v->lds_bytes;
-        state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
-        state->block_dim[0] = (unsigned)v->threads;
-    } else { // the figures of the middle (SpMM) launch
-        state->shared_mem_size = state->spmm.shared_mem_size;
-        state->grid_dim[0] = state->spmm.grid_dim[0];
-        state->block_dim[0] = state->spmm.block_dim[0];
-    }
-    state->grid_dim[1] = state->grid_dim[2] = 1;
-    state->block_dim[1] = state->block_dim[2] = 1;
-    state->init_success = 1;
-    return SHFLBW_OK;
+    const int key[5] = {FORM_PLANES, B, H, W, stride};
+    const int s = stride, copies = g.copies, C = f->C, S = f->S;
+    const long PW = g.PW, pitch = g.pitch;
+    const int *ids = nullptr, *ids_pm = nullptr;
+    // kept-column id k = (r*S + t)*C + c  ->  element offset of (copy, phase, channel) row + tap offset
+    rc = conv_ids_for(fw, key, (int)(g.rows * pitch), [&](int k) {
+        const int c = k % C, tap = k / C, r = tap / S, t = tap % S;
+        const long shift = (long)(r / s) * PW + t / s;
+        const int copy = copies == 2 ? (int)(shift & 1) : 0;
+        const int phase = (r % s) * s + t % s;
+        return (int)((((long)copy * s * s + phase) * C + c) * pitch + shift - copy);
+    }, &ids, &ids_pm);
+    if (rc != SHFLBW_OK) return rc;
+    char* bulk = nullptr;
+    if ((rc = conv_bulk_for(fw, key, IFMap, OFMap, g.planes_bytes + g.dm_bytes, &bulk)) != SHFLBW_OK) return rc;
+    return bind_plane_form(state, f, g, bulk, bulk + g.planes_bytes, ids, ids_pm);
 }
 
-// Forms 4 and 5: phase planes with the batch innermost, planes[phase (a, b)][c][(i * PW + j) * B + img] =
+// XCDs of the current device when it deals the workgroups of a launch to them the way the fused form counts on:
+// consecutive workgroup ids go to consecutive XCDs, round-robin from whichever XCD the launch starts on, so a launch of
+// a multiple of n workgroups puts the same number on every XCD; and every XCD has the same number of compute units.
+// Checked once per device with probe launches of two sizes; 0 when the device deals differently (the fused form is
+// then not offered; `why` says what was seen).
+int device_xcds(std::string* why)
+{
+    static std::mutex lock;
+    static int cached[64] = {}; // 0 = unknown, -1 = not usable
+    static std::string seen[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    std::lock_guard<std::mutex> guard(lock);
+    if (cached[dev] == 0) {
+        cached[dev] = -1;
+        const int sizes[2] = {1024, 256};
+        int* d = nullptr;
+        int n_all = 0;
+        bool ok = hipMalloc((void**)&d, 1024 * sizeof(int)) == hipSuccess;
+        if (!ok) seen[dev] = "probe allocation failed";
+        for (int round = 0; ok && round < 2; round++) {
+            const int blocks = sizes[round];
+            std::vector<int> h(blocks, -1);
+            ok = hipMemset(d, 0xff, blocks * sizeof(int)) == hipSuccess && launch_xcd_probe(d, blocks, nullptr) == hipSuccess &&
+                 hipMemcpy(h.data(), d, blocks * sizeof(int), hipMemcpyDeviceToHost) == hipSuccess;
+            if (!ok) {
+                seen[dev] = "probe launch failed";
+                break;
+            }
+            int n = 0;
+            for (int v : h) n = std::max(n, v + 1);
+            ok = n >= 1 && n <= 8 && (round == 0 || n == n_all) && device_compute_units() % n == 0 && h[0] >= 0;
+            for (int i = 0; ok && i < blocks; i++) ok = h[i] == (h[0] + i) % n;
+            n_all = n;
+            if (!ok) {
+                char buf[256];
+                int len = snprintf(buf, sizeof(buf), "launch of %d workgroups, %d XCD ids, workgroups 0.. ran on XCDs", blocks, n);
+                for (int i = 0; i < 24 && len < (int)sizeof(buf) - 8; i++) len += snprintf(buf + len, sizeof(buf) - len, " %d", h[i]);
+                seen[dev] = buf;
+            }
+        }
+        if (d) (void)hipFree(d);
+        if (ok) cached[dev] = n_all;
+    }
+    if (why) *why = seen[dev];
+    return cached[dev] > 0 ? cached[dev] : 0;
+}
+
+// Geometry of the batch-innermost plane forms (2, 3, 4): phase planes planes[phase (a, b)][c][(i * PW + j) * B + img] =
 // in(i * stride + a - R/2, j * stride + b - S/2) of image img and channel c, PHX = Ho + (R-1)/stride rows and
-// PW = Wo + (S-1)/stride columns.  Every tap offset is a multiple of B values, 16 bytes or more: one copy of the
-// planes serves all taps.  The SpMM runs over the Ho * PW * B columns (ho, j, img) of the padded output grid and
-// drops the padding columns in its epilogue (output_column()).
+// PW = Wo + (S-1)/stride columns.  Every tap offset is a multiple of B values, 16 bytes or more: one copy of the planes
+// serves all taps.  The GEMM runs over the Ho * PW * B columns (ho, j, img) of the padded output grid.
+struct BatchPlanes {
+    int Ho, Wo;
+    long PHX, PW;
+    long np;        // values of one channel plane
+    long rows;      // channel rows: stride^2 * C
+    long ncols;     // columns of the GEMM
+    long max_shift; // largest tap offset in values
+};
+
+void batch_planes_geometry(const shflbw_weight* f, int B, int stride, int Ho, int Wo, BatchPlanes* g)
+{
+    const int s = stride;
+    g->Ho = Ho, g->Wo = Wo;
+    g->PHX = Ho + (f->R - 1) / s;
+    g->PW = Wo + (f->S - 1) / s;
+    g->np = g->PHX * g->PW * B;
+    g->rows = (long)s * s * f->C;
+    g->ncols = (long)Ho * g->PW * B;
+    g->max_shift = ((long)((f->R - 1) / s) * g->PW + (f->S - 1) / s) * B;
+}
+
 //   form 4: the caller's tensors are C-H-W-B / F-H-W-B (the reference's), H and W bound input and output alike,
-//           the SpMM writes OFMap itself;
-//   form 5: the caller's tensors are NHWC with true stride and padding; the SpMM writes result_fm[f][(ho, wo, img)],
+//           the SpMM writes OFMap itself (its epilogue drops the padding columns, output_column());
+//   form 2: the caller's tensors are NHWC with true stride and padding; the SpMM writes result_fm[f][(ho, wo, img)],
 //           a tile transpose writes OFMap.
-static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                             const void* IFMap, void* OFMap, int variant)
+int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                      const void* IFMap, void* OFMap, int variant)
 {
     int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
     if (rc != SHFLBW_OK) return rc;
@@ -659,79 +747,47 @@ static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f,
         return SHFLBW_ERR_UNSUPPORTED;
     }
     SHFLBW_HIP_TRY(k->prepare());
-    if (variant == 4) { // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
+    if (variant == FORM_CHWB) { // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
         state->Ho = H;
         state->Wo = W;
     }
-    const int s = stride, Ho = state->Ho, Wo = state->Wo;
-    const long PHX = Ho + (f->R - 1) / s, PW = Wo + (f->S - 1) / s;
-    const long np = PHX * PW * B;                                  // values of one channel plane
-    const long pitch = (np + (long)((f->S - 1) / s) * B + 8 + 63) / 64 * 64;
-    const long rows = (long)s * s * f->C;
-    const long ncols = (long)Ho * PW * B;                          // columns of the GEMM: the padded output grid
-    if (ncols > 0x7fffffffL || (unsigned long long)(rows + 1) * (unsigned long long)pitch * 2ull > 0xffffffffull) {
-        set_error("spconv_init: problem too large (%ld channel rows of %ld values)", rows, pitch);
+    BatchPlanes g;
+    batch_planes_geometry(f, B, stride, state->Ho, state->Wo, &g);
+    const int s = stride, C = f->C, S = f->S;
+    const long pitch = (g.np + g.max_shift + 8 + 63) / 64 * 64;
+    if (g.ncols > 0x7fffffffL || (unsigned long long)(g.rows + 1) * (unsigned long long)pitch * 2ull > 0xffffffffull) {
+        set_error("spconv_init: problem too large (%ld channel rows of %ld values)", g.rows, pitch);
         return SHFLBW_ERR_UNSUPPORTED;
     }
-    auto up256 = [](size_t n) { return (n + 255) / 256 * 256; };
-    const size_t slots = f->packed_indices.size();
-    const size_t planes_bytes = up256((size_t)(rows + 1) * pitch * 2), ids_bytes = up256(slots * sizeof(int) + 64);
-    const size_t dm_bytes = variant == 5 ? up256((size_t)f->F * Ho * Wo * B * 2) : 0;
-    const size_t total = planes_bytes + dm_bytes + 2 * ids_bytes;
-    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is bookkeeping of the handle (see shflbw_spconv_init_variant)
+    const size_t planes_bytes = up256((size_t)(g.rows + 1) * pitch * 2); // one more row: zeros, for the padding slots
+    const size_t dm_bytes = variant == FORM_BPLANES ? up256((size_t)f->F * g.Ho * g.Wo * B * 2) : 0;
+    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is bookkeeping of the handle (see init_planes)
     std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
-    char* scratch = nullptr;
     const int key[5] = {variant, B, H, W, stride};
-    for (auto& sc : fw->conv_scratch)
-        if (sc.bytes == total && memcmp(sc.key, key, sizeof(key)) == 0 && sc.in == IFMap && sc.out == OFMap)
-            scratch = (char*)sc.ptr;
-    if (!scratch) {
-        void* ptr = nullptr;
-        if (hipMalloc(&ptr, total) != hipSuccess) {
-            set_error("spconv_init: cannot allocate %zu bytes of device scratch", total);
-            return SHFLBW_ERR_HIP;
-        }
-        fw->conv_scratch.push_back(shflbw_weight::Scratch{total, ptr, {variant, B, H, W, stride}, IFMap, OFMap});
-        scratch = (char*)ptr;
-        SHFLBW_HIP_TRY(hipMemset(scratch, 0, planes_bytes)); // includes the row of zeros behind the last channel row
-        // kept-column id k = (r*S + t)*C + c  ->  element offset of the (phase, channel) row + tap offset
-        std::vector<int> ids(slots), ids_pm(slots);
-        for (size_t q = 0; q < slots; q++) {
-            const int kk = f->packed_indices[q];
-            if (kk < 0) {
-                ids[q] = (int)(rows * pitch);
-                continue;
-            }
-            const int c = kk % f->C, tap = kk / f->C, r = tap / f->S, t = tap % f->S;
-            ids[q] = (int)((((long)(r % s) * s + t % s) * f->C + c) * pitch + ((long)(r / s) * PW + t / s) * B);
-        }
-        for (size_t q = 0; q < slots; q++) { // producer-major order inside every 64-slot group
-            const size_t grp = q / 64;
-            const int j = (int)(q % 64) / 16, p = (int)(q % 16) / 4, r = (int)(q % 4);
-            ids_pm[grp * 64 + 16 * p + 4 * j + r] = ids[q];
-        }
-        char* ids_dev = scratch + planes_bytes + dm_bytes;
-        SHFLBW_HIP_TRY(hipMemcpy(ids_dev, ids.data(), slots * sizeof(int), hipMemcpyHostToDevice));
-        SHFLBW_HIP_TRY(hipMemcpy(ids_dev + ids_bytes, ids_pm.data(), slots * sizeof(int), hipMemcpyHostToDevice));
-    }
-    state->planes = scratch;
-    state->result_fm = variant == 5 ? scratch + planes_bytes : nullptr;
-    state->np = (int)np;
-    state->plane_rows = (int)PHX;
-    state->plane_cols = (int)PW;
+    const long PW = g.PW;
+    const int *ids = nullptr, *ids_pm = nullptr;
+    // kept-column id k = (r*S + t)*C + c  ->  element offset of the (phase, channel) row + tap offset
+    rc = conv_ids_for(fw, key, (int)(g.rows * pitch), [&](int kk) {
+        const int c = kk % C, tap = kk / C, r = tap / S, t = tap % S;
+        return (int)((((long)(r % s) * s + t % s) * C + c) * pitch + ((long)(r / s) * PW + t / s) * B);
+    }, &ids, &ids_pm);
+    if (rc != SHFLBW_OK) return rc;
+    char* bulk = nullptr;
+    if ((rc = conv_bulk_for(fw, key, IFMap, OFMap, planes_bytes + dm_bytes, &bulk)) != SHFLBW_OK) return rc;
+    state->planes = bulk;
+    state->result_fm = variant == FORM_BPLANES ? bulk + planes_bytes : nullptr;
+    state->np = (int)g.np;
+    state->plane_rows = (int)g.PHX;
+    state->plane_cols = (int)g.PW;
     state->plane_pitch = (int)pitch;
     state->plane_copies = 1;
-    state->ncols = (int)ncols;
+    state->ncols = (int)g.ncols;
     // the SpMM in the middle: row f of its result is the row of filter f, in OFMap itself (form 4) or in result_fm
-    rc = shflbw_spmm_init_variant(&state->spmm, f, (int)ncols, state->planes, nullptr,
-                                  variant == 5 ? state->result_fm : OFMap, 1.f, 0.f, 0);
+    rc = bind_middle(state, f, g.ncols, state->planes, variant == FORM_BPLANES ? state->result_fm : OFMap, ids, ids_pm,
+                     (g.rows + 1) * pitch);
     if (rc != SHFLBW_OK) return rc;
-    state->spmm.packed_indices = (const int*)(scratch + planes_bytes + dm_bytes);
-    state->spmm.packed_indices_pm = (const int*)(scratch + planes_bytes + dm_bytes + ids_bytes);
-    state->spmm.ldb_bytes = 2;
-    state->spmm.args.K = (int)((rows + 1) * pitch);
     state->shared_mem_size = (size_t)k->lds_bytes;
-    state->grid_dim[0] = (unsigned)((f->nrow / f->brow) * ((ncols + k->BN - 1) / k->BN));
+    state->grid_dim[0] = (unsigned)((f->nrow / f->brow) * ((g.ncols + k->BN - 1) / k->BN));
     state->block_dim[0] = (unsigned)k->threads;
     state->grid_dim[1] = state->grid_dim[2] = 1;
     state->block_dim[1] = state->block_dim[2] = 1;
@@ -739,21 +795,103 @@ static int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f,
     return SHFLBW_OK;
 }
 
-int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
-                            const void* IFMap, void* OFMap)
+// Layout of the fused form's bulk scratch: nx slabs of planes | nx filter-major results | counters.
+struct FusedForm {
+    BatchPlanes g;
+    int nx;          // XCDs of the device
+    long cx;         // columns of the GEMM per XCD (a multiple of 64)
+    long pitch;      // values per channel row of a slab: cx + the largest tap offset, rounded up to 64
+    size_t slab_bytes, fm_bytes, sync_bytes;
+    size_t total_bytes() const { return (size_t)nx * (slab_bytes + fm_bytes) + sync_bytes; }
+};
+
+int fused_form_geometry(const shflbw_weight* f, int B, int stride, int Ho, int Wo, int nx, FusedForm* g)
 {
-    return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, 4);
+    batch_planes_geometry(f, B, stride, Ho, Wo, &g->g);
+    g->nx = nx;
+    g->cx = ((g->g.ncols + nx - 1) / nx + 63) / 64 * 64;
+    g->pitch = (g->cx + g->g.max_shift + 63) / 64 * 64;
+    if (stride * stride > 32 || g->g.ncols > 0x7fffffffL ||
+        (unsigned long long)(g->g.rows + 1) * (unsigned long long)g->pitch * 2ull > 0x7fffffffull ||
+        (unsigned long long)f->F * (unsigned long long)g->cx > 0x7fffffffull) {
+        set_error("spconv_init: problem too large for the fused form (%ld channel rows of %ld values per XCD)", g->g.rows, g->pitch);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    g->slab_bytes = up256((size_t)(g->g.rows + 1) * g->pitch * 2); // one more row: zeros, for the padding slots
+    g->fm_bytes = up256((size_t)f->F * g->cx * 2);
+    g->sync_bytes = (size_t)conv_xcd_sync_lines(nx) * SYNC_LINE * sizeof(int);
+    return SHFLBW_OK;
 }
 
-int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
+// form 3: NHWC tensors, the three steps of form 2 in one launch, every XCD on its own columns (spconv_xcd_kernel)
+int init_fused(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride, const void* IFMap,
+               void* OFMap)
 {
-    if (!state || !state->init_success) {
-        set_error("spconv_exec: state was not initialised successfully");
-        return SHFLBW_ERR_STATE;
+    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, FORM_FUSED);
+    if (rc != SHFLBW_OK) return rc;
+    if (B % 8 != 0) {
+        set_error("spconv_init: the batch must be a multiple of 8 for this form (got %d)", B);
+        return SHFLBW_ERR_SHAPE;
     }
-    const SpconvVariant* v = find_spconv_variant(state->brow, 0, nullptr); // the direct kernel of this block size
-    if (!v && state->variant == 1) return SHFLBW_ERR_UNSUPPORTED;
-    SpconvLaunchArgs a;
+    const ConvXcdKernel* k = conv_xcd_kernel(f->brow);
+    if (!k) {
+        set_error("spconv_init: no fused kernel for block size %d", f->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    std::string why;
+    const int nx = device_xcds(&why);
+    if (nx <= 0) {
+        set_error("spconv_init: this device does not deal workgroups to its XCDs in the way the fused form counts on (%s)", why.c_str());
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    if (device_compute_units() / nx > 32) {
+        set_error("spconv_init: the fused form numbers at most 32 workgroups per XCD (this device: %d)", device_compute_units() / nx);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    SHFLBW_HIP_TRY(k->prepare());
+    FusedForm g;
+    if ((rc = fused_form_geometry(f, B, stride, state->Ho, state->Wo, nx, &g)) != SHFLBW_OK) return rc;
+    const int s = stride, C = f->C, S = f->S;
+    const long PW = g.g.PW, pitch = g.pitch;
+    shflbw_weight* fw = const_cast<shflbw_weight*>(f); // the scratch cache is bookkeeping of the handle (see init_planes)
+    std::lock_guard<std::mutex> scratch_guard(fw->scratch_lock);
+    const int key[5] = {FORM_FUSED, B, H, W, stride};
+    const int *ids = nullptr, *ids_pm = nullptr;
+    // kept-column id k = (r*S + t)*C + c  ->  element offset inside a slab: (phase, channel) row + tap offset
+    rc = conv_ids_for(fw, key, (int)(g.g.rows * pitch), [&](int kk) {
+        const int c = kk % C, tap = kk / C, r = tap / S, t = tap % S;
+        return (int)((((long)(r % s) * s + t % s) * C + c) * pitch + ((long)(r / s) * PW + t / s) * B);
+    }, &ids, &ids_pm);
+    if (rc != SHFLBW_OK) return rc;
+    char* bulk = nullptr;
+    if ((rc = conv_bulk_for(fw, key, IFMap, OFMap, g.total_bytes(), &bulk)) != SHFLBW_OK) return rc;
+    state->planes = bulk;
+    state->result_fm = bulk + (size_t)nx * g.slab_bytes;
+    state->sync = bulk + (size_t)nx * (g.slab_bytes + g.fm_bytes);
+    state->np = (int)g.g.np;
+    state->plane_rows = (int)g.g.PHX;
+    state->plane_cols = (int)g.g.PW;
+    state->plane_pitch = (int)pitch;
+    state->plane_copies = 1;
+    state->ncols = (int)g.g.ncols;
+    state->xcds = nx;
+    state->cols_per_xcd = (int)g.cx;
+    // the SpMM in the middle, as one XCD sees it: cx columns, its slab as B, its result as D
+    rc = bind_middle(state, f, g.cx, state->planes, state->result_fm, ids, ids_pm, (g.g.rows + 1) * pitch);
+    if (rc != SHFLBW_OK) return rc;
+    state->shared_mem_size = (size_t)k->lds_bytes;
+    state->grid_dim[0] = (unsigned)(device_compute_units() / nx * nx);
+    state->block_dim[0] = (unsigned)k->threads;
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
+// launch arguments every form shares
+void fill_conv_launch_args(const shflbw_spconv_state* state, SpconvLaunchArgs* out)
+{
+    SpconvLaunchArgs& a = *out;
     a.B = state->args.B;
     a.H = state->args.H;
     a.W = state->args.W;
@@ -774,15 +912,83 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     a.row_ids = state->args.A_row_indices;
     a.in = (const half_t*)state->args.IFMap;
     a.out = (half_t*)state->args.OFMap;
-    if (state->variant == 4 || state->variant == 5) {
+}
+
+// Chunks of the layout phases of the fused form: `tiles` = 8, 4 or 2 tiles of 64 x 64 per chunk, as many of them
+// along the contiguous axis of the source (`along` tiles there) as there are.  Picks the chunk size that needs the
+// fewest rounds of the `workers` workgroups of an XCD, a round costing its tiles plus a fixed latency of about
+// four tiles' worth.
+void pick_chunk(int along_tiles, int across_tiles, int workers, int* t_along, int* t_across, int* chunks_along)
+{
+    auto pow2_le = [](int n, int cap) { int p = 1; while (p * 2 <= n && p * 2 <= cap) p *= 2; return p; };
+    long best_cost = -1;
+    for (int tiles = 8; tiles >= 2; tiles >>= 1) {
+        const int ta = pow2_le(along_tiles, tiles), tb = tiles / ta;
+        const long chunks = (long)((along_tiles + ta - 1) / ta) * ((across_tiles + tb - 1) / tb);
+        const long rounds = (chunks + workers - 1) / workers;
+        const long cost = rounds * (tiles + 4);
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            *t_along = ta, *t_across = tb, *chunks_along = (along_tiles + ta - 1) / ta;
+        }
+    }
+}
+
+} // namespace
+
+extern "C" {
+
+int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                               const void* IFMap, void* OFMap, int variant)
+{
+    if (variant == FORM_CHWB) {
+        if (state) memset(state, 0, sizeof(*state));
+        set_error("spconv_init: form 4 works on C-H-W-B / F-H-W-B tensors; call shflbw_spconv_init_chwb");
+        return SHFLBW_ERR_INVALID;
+    }
+    // the library's choice: a batch-innermost form where the batch allows it (one copy of the planes instead of two, no
+    // dead plane rows in the result), else the plane form
+    if (variant < 0) variant = B > 0 && B % 8 == 0 ? FORM_BPLANES : FORM_PLANES;
+    if (variant == FORM_BPLANES) return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, FORM_BPLANES);
+    if (variant == FORM_FUSED) return init_fused(state, f, B, H, W, stride, IFMap, OFMap);
+    if (variant == FORM_PLANES) return init_planes(state, f, B, H, W, stride, IFMap, OFMap);
+    int rc = spconv_fill_state(state, f, B, H, W, stride, IFMap, OFMap, variant);
+    if (rc != SHFLBW_OK) return rc;
+    // the direct kernel
+    const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
+    const long npix = (long)B * state->Ho * state->Wo;
+    state->shared_mem_size = (size_t)v->lds_bytes;
+    state->grid_dim[0] = (unsigned)((f->F / f->brow) * ((npix + v->BN - 1) / v->BN));
+    state->block_dim[0] = (unsigned)v->threads;
+    state->grid_dim[1] = state->grid_dim[2] = 1;
+    state->block_dim[1] = state->block_dim[2] = 1;
+    state->init_success = 1;
+    return SHFLBW_OK;
+}
+
+int shflbw_spconv_init_chwb(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H, int W, int stride,
+                            const void* IFMap, void* OFMap)
+{
+    return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, FORM_CHWB);
+}
+
+int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
+{
+    if (!state || !state->init_success) {
+        set_error("spconv_exec: state was not initialised successfully");
+        return SHFLBW_ERR_STATE;
+    }
+    SpconvLaunchArgs a;
+    fill_conv_launch_args(state, &a);
+    hipError_t e = hipSuccess;
+    if (state->variant == FORM_CHWB || state->variant == FORM_BPLANES) {
         const ConvChwbKernel* k = conv_chwb_kernel(state->brow);
         if (!k) return SHFLBW_ERR_UNSUPPORTED;
-        const bool nhwc = state->variant == 5;
-        hipError_t e = nhwc ? launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
-                                                    state->plane_pitch, 1, (hipStream_t)stream, 1)
-                            : launch_chwb_to_planes(a.in, (half_t*)state->planes, a.B, a.H, a.W, a.C, a.R, a.S, a.stride,
-                                                    state->plane_rows, state->plane_cols, state->plane_pitch,
-                                                    (hipStream_t)stream);
+        const bool nhwc = state->variant == FORM_BPLANES;
+        e = nhwc ? launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
+                                         state->plane_pitch, 1, (hipStream_t)stream, 1)
+                 : launch_chwb_to_planes(a.in, (half_t*)state->planes, a.B, a.H, a.W, a.C, a.R, a.S, a.stride,
+                                         state->plane_rows, state->plane_cols, state->plane_pitch, (hipStream_t)stream);
         SpmmLaunchArgs m;
         fill_spmm_launch_args(&state->spmm, k->BN, &m);
         m.alternate = 0;
@@ -794,117 +1000,76 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         if (e == hipSuccess && nhwc) // result_fm[f][(ho, wo, img)] -> OFMap[img][ho][wo][f]
             e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, a.Ho * a.Wo * a.B, a.B, a.Ho, a.Wo,
                                       a.Ho, a.Wo, (hipStream_t)stream, 1);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
-        }
-        return SHFLBW_OK;
-    }
-    if (state->variant == 3) {
-        const ConvFusedKernel* k = conv_fused_kernel(state->brow);
-        if (!k) return SHFLBW_ERR_UNSUPPORTED;
+    } else if (state->variant == FORM_FUSED) {
+        const ConvXcdKernel* k = conv_xcd_kernel(state->brow);
+        if (!k || state->xcds <= 0 || state->cols_per_xcd <= 0) return SHFLBW_ERR_UNSUPPORTED;
         SpmmLaunchArgs m;
         fill_spmm_launch_args(&state->spmm, k->BN, &m);
         if (m.X == 0) return SHFLBW_OK;
-        m.alternate = 0; // the planes under one column tile are far smaller than an L2
-        m.img_cols = a.Ho * state->plane_cols;
-        m.img_skip = (state->plane_rows - a.Ho) * state->plane_cols;
-        m.tile_arrivals = (int*)state->sync + CONV_LINE_SLAB0 * SYNC_LINE;
-        ConvFuseArgs c;
-        c.g = PlaneGeom{a.B, a.H, a.W, a.C, a.stride, a.pad_h, a.pad_w, state->plane_rows, state->plane_cols,
-                        state->plane_pitch, state->plane_copies, 0, {}};
+        m.alternate = 0; // a slab is far smaller than an L2
+        m.ldd = state->cols_per_xcd;
+        const int s = a.stride, nx = state->xcds, cx = state->cols_per_xcd;
+        ConvXcdArgs c;
+        c.g = PlaneGeom{a.B, a.H, a.W, a.C, s, a.pad_h, a.pad_w, state->plane_rows, state->plane_cols, state->plane_pitch, 1, 0, {}, 1};
         if (!fill_wanted_planes(c.g, a.R, a.S)) return SHFLBW_ERR_UNSUPPORTED;
-        // chunks of the two layout phases: 8, 4 or 2 tiles of 64 x 64, the largest size that still gives every
-        // workgroup a chunk; along the contiguous axis of the source (channels, filters) as many tiles as there are
-        auto pow2_le = [](int n, int cap) { int p = 1; while (p * 2 <= n && p * 2 <= cap) p *= 2; return p; };
-        const int grid = std::min((m.num_cus / 8) * 8, ((m.X * ((state->ncols + k->BN - 1) / k->BN) + 7) / 8) * 8);
         c.in = a.in;
-        c.planes = (half_t*)state->planes;
-        c.np64 = (state->np + 63) / 64 * 64;
-        for (int tiles = 8; tiles >= 2; tiles >>= 1) {
-            c.ct = pow2_le((a.C + 63) / 64, tiles);
-            c.pt = tiles / c.ct;
-            c.ch_chunks = (a.C + c.ct * 64 - 1) / (c.ct * 64);
-            c.pos_chunks = (c.np64 + c.pt * 64 - 1) / (c.pt * 64);
-            c.n0chunks = c.g.nwanted * c.ch_chunks * c.pos_chunks;
-            if (c.n0chunks >= grid) break;
-        }
-        c.fm = (const half_t*)state->result_fm;
         c.out = a.out;
-        c.F = a.F;
-        c.ncols = state->ncols;
-        c.Ho = a.Ho;
-        c.Wo = a.Wo;
-        for (int tiles = 8; tiles >= 2; tiles >>= 1) {
-            c.ft = pow2_le((a.F + 63) / 64, tiles);
-            c.mt = tiles / c.ft;
-            c.f_chunks = (a.F + c.ft * 64 - 1) / (c.ft * 64);
-            if (c.f_chunks * ((k->BN / 64 + c.mt - 1) / c.mt) >= m.X) break; // a chunk for every workgroup of a column tile
-        }
-        c.slabs = (state->ncols + k->BN - 1) / k->BN;
-        c.arrivals_per_slab = m.X;
+        c.nx = nx, c.cx = cx, c.ncols = state->ncols;
+        c.max_shift = (((a.R - 1) / s) * state->plane_cols + (a.S - 1) / s) * a.B;
+        c.slabs = (half_t*)state->planes;
+        c.slab_elems = up256((size_t)(s * s * a.C + 1) * state->plane_pitch * 2) / 2;
+        c.fm = (half_t*)state->result_fm;
+        c.fm_elems = up256((size_t)a.F * cx * 2) / 2;
         c.sync = (int*)state->sync;
-        c.magic_ps = udiv_magic(state->plane_rows * state->plane_cols);
+        c.F = a.F, c.Ho = a.Ho, c.Wo = a.Wo;
+        const int workers = std::max(1, m.num_cus / nx);
+        const int n_x = std::min(cx, state->ncols); // the columns of a full XCD
+        pick_chunk((a.C + 63) / 64, (n_x + c.max_shift + 63) / 64 * c.g.nwanted, workers, &c.ct, &c.pt, &c.ch_chunks);
+        pick_chunk((a.F + 63) / 64, (n_x + 63) / 64, workers, &c.ft, &c.mt, &c.f_chunks);
+        c.magic_b = udiv_magic(a.B);
         c.magic_pw = udiv_magic(state->plane_cols);
-        c.magic_imgcols = udiv_magic(a.Ho * state->plane_cols);
-        c.help_ticks = 3000; // 30 us
-        // Measurement knob: SHFLBW_FUSED_PHASES (bit 0: input rewrite inside the launch, bit 1: NHWC output inside
-        // the launch; default 3).  A cleared bit runs that step as its own launch around the fused kernel.
-        static const int phases = [] {
-            const char* e = getenv("SHFLBW_FUSED_PHASES");
-            return e ? atoi(e) & 3 : 3;
-        }();
-        c.phases = phases;
-        hipError_t e = hipSuccess;
-        if (!(phases & 1))
-            e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols, state->plane_pitch,
-                                      state->plane_copies, (hipStream_t)stream);
-        if (e == hipSuccess) e = k->launch(m, c, (hipStream_t)stream);
-        if (e == hipSuccess && !(phases & 2)) // the compact result has Ho rows per image
-            e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, state->ncols, a.B, a.Ho,
+        c.spin_ticks = 20000000; // 0.2 s
+        c.patience = 5000;       // 50 us
+        c.debug = 0;
+#ifdef SHFLBW_CONV_STAMPS
+        if (const char* dbg = getenv("SHFLBW_CONV_DEBUG")) c.debug = atoi(dbg);
+#endif
+        e = k->launch(m, c, (hipStream_t)stream);
+    } else if (state->variant == FORM_PLANES) {
+        e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols, state->plane_pitch,
+                                  state->plane_copies, (hipStream_t)stream);
+        if (e == hipSuccess) {
+            int rc = shflbw_spmm_exec(&state->spmm, stream);
+            if (rc != SHFLBW_OK) return rc;
+            e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, state->np, a.B, state->plane_rows,
                                       state->plane_cols, a.Ho, a.Wo, (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: fused launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
         }
-        return SHFLBW_OK;
+    } else {
+        const SpconvVariant* v = find_spconv_variant(state->brow, 0, nullptr); // the direct kernel of this block size
+        if (!v) return SHFLBW_ERR_UNSUPPORTED;
+        e = v->launch(a, (hipStream_t)stream);
     }
-    if (state->variant == 0) {
-        hipError_t e = launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,
-                                             state->plane_pitch, state->plane_copies, (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: plane layout launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
-        }
-        int rc = shflbw_spmm_exec(&state->spmm, stream);
-        if (rc != SHFLBW_OK) return rc;
-        e = launch_planes_to_nhwc((const half_t*)state->result_fm, a.out, a.F, state->np, a.B, state->plane_rows,
-                                  state->plane_cols, a.Ho, a.Wo, (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: transpose launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
-        }
-        return SHFLBW_OK;
-    }
-    if (state->variant == 2) {
-        hipError_t e = launch_im2col_nhwc(a, (half_t*)state->im2col, state->np, (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: im2col launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
-        }
-        int rc = shflbw_spmm_exec(&state->spmm, stream);
-        if (rc != SHFLBW_OK) return rc;
-        e = launch_transpose_to_nhwc((const half_t*)state->result_fm, a.out, a.F, a.B * a.Ho * a.Wo, state->np,
-                                     (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("spconv_exec: transpose launch failed: %s", hipGetErrorString(e));
-            return SHFLBW_ERR_HIP;
-        }
-        return SHFLBW_OK;
-    }
-    hipError_t e = v->launch(a, (hipStream_t)stream);
     if (e != hipSuccess) {
         set_error("spconv_exec: launch failed: %s", hipGetErrorString(e));
+        return SHFLBW_ERR_HIP;
+    }
+    return SHFLBW_OK;
+}
+
+int shflbw_spconv_check(const shflbw_spconv_state* state)
+{
+    if (!state || !state->init_success) {
+        set_error("spconv_check: state was not initialised successfully");
+        return SHFLBW_ERR_STATE;
+    }
+    if (state->variant != FORM_FUSED) return SHFLBW_OK;
+    int flag = 0;
+    SHFLBW_HIP_TRY(hipMemcpy(&flag, state->sync, sizeof(int), hipMemcpyDeviceToHost)); // waits for the device
+    if (flag != 0) {
+        // leave the scratch as a fresh one: no counter may keep what the failed launch left in it
+        SHFLBW_HIP_TRY(hipMemset(state->sync, 0, (size_t)conv_xcd_sync_lines(state->xcds) * SYNC_LINE * sizeof(int)));
+        set_error(flag == 1 ? "spconv_check: the workgroups of a fused launch were not dealt to the XCDs the way init had checked; results are invalid"
+                            : "spconv_check: a wait between the phases of the fused form ran out of time; results are invalid");
         return SHFLBW_ERR_HIP;
     }
     return SHFLBW_OK;
@@ -953,7 +1118,7 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
                               void* stream)
 {
     shflbw_spconv_state st;
-    int rc = spconv_fill_state(&st, f, B, H, W, stride, IFMap, OFMap, 0);
+    int rc = spconv_fill_state(&st, f, B, H, W, stride, IFMap, OFMap, FORM_PLANES);
     if (rc != SHFLBW_OK) return rc;
     PlaneForm g;
     if ((rc = plane_form_geometry(f, B, H, W, stride, &g)) != SHFLBW_OK) return rc;
@@ -966,11 +1131,11 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
     if ((rc = static_scratch_address(&base)) != SHFLBW_OK) return rc;
     // Nothing in the array has to start at zero: the layout pass writes every plane position a pixel's taps
     // read (zeros outside the image), the rest only feeds plane positions that are no output pixel.
-    if ((rc = bind_plane_form(&st, f, g, base, false)) != SHFLBW_OK) return rc;
-    hipError_t e = launch_plane_ids((const int*)f->d_packed_indices, (int*)(base + g.planes_bytes + g.dm_bytes),
-                                    (int*)(base + g.planes_bytes + g.dm_bytes + g.ids_bytes), (int)g.slots, f->C, f->S,
-                                    stride, g.PW, (int)g.pitch, g.copies, (int)(g.rows * g.pitch), (half_t*)base,
-                                    (hipStream_t)stream);
+    int* ids = (int*)(base + g.planes_bytes + g.dm_bytes);
+    int* ids_pm = (int*)(base + g.planes_bytes + g.dm_bytes + g.ids_bytes);
+    if ((rc = bind_plane_form(&st, f, g, base, base + g.planes_bytes, ids, ids_pm)) != SHFLBW_OK) return rc;
+    hipError_t e = launch_plane_ids((const int*)f->d_packed_indices, ids, ids_pm, (int)g.slots, f->C, f->S, stride, g.PW,
+                                    (int)g.pitch, g.copies, (int)(g.rows * g.pitch), (half_t*)base, (hipStream_t)stream);
     if (e != hipSuccess) {
         set_error("spconv_exec_static: id launch failed: %s", hipGetErrorString(e));
         return SHFLBW_ERR_HIP;
@@ -978,29 +1143,39 @@ int shflbw_spconv_exec_static(const shflbw_weight* f, int B, int H, int W, int s
     return shflbw_spconv_exec(&st, stream);
 }
 
-static const char* const g_spconv_forms[] = {
+static const char* const g_spconv_forms[FORM_COUNT] = {
     "planes+spmm+transpose",  // 0: NHWC -> channel-major planes, SpMM gather with tap offsets, transpose to NHWC: three launches
     "direct",                 // 1: one kernel, im2col gather from NHWC in the tile loads
-    "im2col+spmm+transpose",  // 2: explicit im2col matrix, three launches
-    "fused-planes",           // 3: the steps of form 0 in one persistent launch
+    "bplanes+spmm+transpose", // 2: NHWC tensors, planes and result with the batch innermost (batch a multiple of 8): three launches
+    "bplanes-fused",          // 3: the steps of form 2 in one persistent launch, every XCD on its own columns
     "chwb-planes+spmm",       // 4: the reference's batch-innermost tensors (shflbw_spconv_init_chwb only): padded copy, SpMM
-    "bplanes+spmm+transpose", // 5: NHWC tensors, planes and result with the batch innermost (batch a multiple of 8): three launches
 };
 
-int shflbw_spconv_variant_count(void) { return (int)(sizeof(g_spconv_forms) / sizeof(g_spconv_forms[0])); }
+int shflbw_spconv_variant_count(void) { return FORM_COUNT; }
 
 const char* shflbw_spconv_variant_name(int variant)
 {
-    return variant >= 0 && variant < shflbw_spconv_variant_count() ? g_spconv_forms[variant] : "";
+    return variant >= 0 && variant < FORM_COUNT ? g_spconv_forms[variant] : "";
 }
 
 int shflbw_weight_release_scratch(shflbw_weight* w)
 {
     if (!w) return SHFLBW_ERR_INVALID;
     std::lock_guard<std::mutex> guard(w->scratch_lock);
-    for (auto& sc : w->conv_scratch)
-        if (sc.ptr) (void)hipFree(sc.ptr);
-    w->conv_scratch.clear();
+    release_conv_scratch(w);
+    return SHFLBW_OK;
+}
+
+int shflbw_weight_scratch_bytes(const shflbw_weight* w, size_t* bytes, int* buffers)
+{
+    if (!w) return SHFLBW_ERR_INVALID;
+    shflbw_weight* fw = const_cast<shflbw_weight*>(w);
+    std::lock_guard<std::mutex> guard(fw->scratch_lock);
+    size_t total = 0;
+    for (auto& e : w->conv_ids) total += e.bytes;
+    for (auto& e : w->conv_bulk) total += e.bytes;
+    if (bytes) *bytes = total;
+    if (buffers) *buffers = (int)(w->conv_ids.size() + w->conv_bulk.size());
     return SHFLBW_OK;
 }
 

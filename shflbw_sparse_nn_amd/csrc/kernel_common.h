@@ -84,19 +84,54 @@ __device__ __forceinline__ void wait_vmcnt_fence()
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// 16-byte store of result values with device scope: the line is written through to memory instead of
-// staying dirty in the XCD's L2, where its later eviction would fall into the gathers of the next tile.
-// The compiler has no form of this store, so it is inline assembly, and the compiler's hazard pass does
-// not look inside: a vector-ALU write to the data registers directly behind a store of more than 8 bytes
-// needs wait states, which the s_nop supplies (the registers are free for reuse after the statement).
+// 16-byte store of result values.
+// DEVICE_SCOPE (the SpMM proper): the line is written through to memory instead of staying dirty in the XCD's L2,
+// where its later eviction would fall into the gathers of the next tile.  The compiler has no form of this store,
+// so it is inline assembly, and the compiler's hazard pass does not look inside: a vector-ALU write to the data
+// registers directly behind a store of more than 8 bytes needs wait states, which the s_nop supplies (the
+// registers are free for reuse after the statement).
+// Otherwise (results that workgroups of the same XCD read back in the same launch): an ordinary store, the line
+// stays in the XCD's L2.
+template <bool DEVICE_SCOPE = true>
 __device__ __forceinline__ void store_result_16B(half_t* p, half8_t v)
 {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    if constexpr (DEVICE_SCOPE)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else
+        asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
 // Words that workgroups of one launch count in (queues, arrival counts) are kept one cache line apart: atomics on
 // one line are served one after the other (about 11 ns each with every compute unit taking part).
 constexpr int SYNC_LINE = 64; // ints
+
+// Counting between the workgroups of ONE XCD.  The compute units of an XCD share its L2, where every atomic is
+// executed; these atomics carry no device scope, so they stay in that L2 instead of going to memory (about 220 ns a
+// round trip on an idle chip; atomics on one cache line are served one after the other, about 11 ns each).  Only
+// workgroups that run on the same XCD may use a given word.  The read is an atomic too (maximum with a value below
+// every count): an atomic is never served by the compute unit's own cache, and a load that carries device scope,
+// which is not either, turned out slower than the atomic once the line is being counted in (the waits of the
+// fused convolution took 3.0 instead of 1.8 us with it).
+__device__ __forceinline__ int xcd_fetch_add(int* p, int v)
+{
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ int xcd_fetch_or(int* p, int v)
+{
+    return __hip_atomic_fetch_or(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ int xcd_read(int* p)
+{
+    return __hip_atomic_fetch_max(p, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// the XCD this wave runs on (0 .. 7 on an MI355X in its single-partition mode)
+__device__ __forceinline__ int xcd_id()
+{
+    unsigned v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    return (int)(v & 15u);
+}
 
 // n / d and n % d for n < 2^31 with magic = floor(2^32 / d) computed on the host (udiv_magic below): the product's high word
 // is the quotient or one less, one correction step settles it; an integer division by a run-time value costs about

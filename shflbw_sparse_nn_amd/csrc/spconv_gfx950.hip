@@ -158,16 +158,6 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
 }
 
 
-// =======================================================================================
-// im2col form of the convolution: three launches on the caller's stream
-//   1. im2col_nhwc_kernel:   NHWC input -> im2col matrix Bm[k][p], k = (r,s,c), p = output pixel,
-//                            rows of NP fp16 (NP = pixel count rounded up to 64), zero outside the image
-//   2. the SpMM kernel:      Dm[f][p] = A_sparse * Bm (row permutation applied to f)
-//   3. transpose_to_nhwc_kernel: Dm[f][p] -> OFMap[p][f]
-// The gather that the sparse filter needs is a gather of whole rows of a [k][pixel] matrix; NHWC
-// keeps channels, not pixels, contiguous, and a row-permuted filter scatters its output channels,
-// so both ends are turned into plain 64 x 64 tile transposes and the middle is the tuned SpMM.
-// =======================================================================================
 constexpr int TT = 64; // transpose tile edge
 
 // 256 threads move a 64 x 64 fp16 tile: `load(i, j)` returns the 16-byte piece j (8 halves) of source
@@ -193,82 +183,6 @@ __device__ __forceinline__ void transpose_tile_64(half_t (*tile)[TT], Load load,
         for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][c];
         store(o, q, v);
     }
-}
-
-// grid: (pixel tiles, channel tiles, filter rows r); block 256.  A workgroup walks the S taps of its
-// filter row: the pixel decode is done once, and the loads of the next tap are in flight while the
-// current one goes through LDS.
-__global__ void __launch_bounds__(256) im2col_nhwc_kernel(const half_t* __restrict__ in, half_t* __restrict__ bm, int B,
-                                                          int H, int W, int C, int S, int stride, int pad_h, int pad_w,
-                                                          int Ho, int Wo, int NP)
-{
-    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
-    const int t = threadIdx.x;
-    const int p0 = blockIdx.x * TT, c0 = blockIdx.y * TT, r = blockIdx.z;
-    const int npix = B * Ho * Wo;
-    // the two source pieces of this thread: pixels p0 + i, channels c0 + 8j ..
-    const int j = t & 7, c = c0 + j * 8;
-    long base[2]; // element offset of (b, hi, wi = wo*stride - pad_w, c)
-    bool row_ok[2]; // the input row hi exists
-    int wi0[2];
-#pragma unroll
-    for (int pass = 0; pass < 2; pass++) {
-        const int p = p0 + (t >> 3) + pass * 32;
-        const int wo = p % Wo, ho = (p / Wo) % Ho, b = p / (Wo * Ho);
-        const int hi = ho * stride - pad_h + r;
-        wi0[pass] = wo * stride - pad_w;
-        row_ok[pass] = p < npix && c < C && hi >= 0 && hi < H;
-        base[pass] = ((long)(b * H + hi) * W + wi0[pass]) * C + c;
-    }
-    auto fetch = [&](int s, int pass) {
-        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-        const int wi = wi0[pass] + s;
-        if (row_ok[pass] && wi >= 0 && wi < W) v = *(const half8_t*)(in + base[pass] + (long)s * C);
-        return v;
-    };
-    half8_t nxt[2] = {fetch(0, 0), fetch(0, 1)};
-    for (int s = 0; s < S; s++) {
-#pragma unroll
-        for (int pass = 0; pass < 2; pass++) {
-            const int i = (t >> 3) + pass * 32;
-            *(half8_t*)&tile[i][(j ^ ((i >> 3) & 7)) * 8] = nxt[pass];
-        }
-        __syncthreads();
-        if (s + 1 < S) {
-            nxt[0] = fetch(s + 1, 0);
-            nxt[1] = fetch(s + 1, 1);
-        }
-        const int tap = r * S + s;
-#pragma unroll
-        for (int pass = 0; pass < 2; pass++) {
-            const int o = (t >> 3) + pass * 32, q = t & 7;
-            const int col = (((o >> 3) ^ q) << 3) | (o & 7);
-            half8_t v;
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = tile[q * 8 + e][col];
-            if (c0 + o < C) *(half8_t*)(bm + ((size_t)tap * C + c0 + o) * NP + p0 + q * 8) = v;
-        }
-        __syncthreads();
-    }
-}
-
-// grid: (pixel tiles, filter tiles); block 256
-__global__ void __launch_bounds__(256) transpose_to_nhwc_kernel(const half_t* __restrict__ dm, half_t* __restrict__ out,
-                                                                int F, int npix, int NP)
-{
-    __shared__ __attribute__((aligned(16))) half_t tile[TT][TT];
-    const int p0 = blockIdx.x * TT, f0 = blockIdx.y * TT;
-    transpose_tile_64(
-        tile,
-        [&](int i, int j) { // source row = filter f0 + i, piece = pixels p0 + 8j ..
-            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (f0 + i < F) v = *(const half8_t*)(dm + (size_t)(f0 + i) * NP + p0 + j * 8);
-            return v;
-        },
-        [&](int o, int q, half8_t v) { // destination row = pixel p0 + o, filters f0 + 8q ..
-            const int pix = p0 + o, f = f0 + q * 8;
-            if (pix < npix && f < F) *(half8_t*)(out + (size_t)pix * F + f) = v;
-        });
 }
 
 // =======================================================================================
@@ -357,49 +271,6 @@ bool fill_wanted_planes(PlaneGeom& g, int R, int S)
     return true;
 }
 
-// =======================================================================================
-// Fused form of the convolution: ONE persistent launch.
-//   phase 0  every workgroup takes chunks of the NHWC -> planes rewrite from a queue (64 x 64 tile transposes,
-//            eight tiles at a time) until the queue is empty, then waits until all chunks have been written;
-//   phase 1  the role-split SpMM over its tiles (gather ids are plane offsets; the columns of the GEMM are the
-//            plane positions of output rows only: m = (img * Ho + i) * PW + j), result rows of fp16 in the
-//            filter-major scratch fm[f][m]; every consumer wave counts its finished tile in the arrival word of
-//            the tile's column tile;
-//   phase 2  when all tiles of a column tile have arrived, its fm[F][BN] slab is transposed to NHWC in chunks
-//            taken from that column tile's queue.
-// No wait depends on a workgroup that is not running: phase 0 waits only for chunks that running workgroups
-// have claimed; in phase 2 the workgroup whose arrival completes a column tile finds it complete when it gets
-// there and empties its queue (alone, if it must), every other wait is bounded by a time budget and only adds
-// helpers.  The words in `sync` are all zero between launches: the last workgroup to leave clears them.
-// Data written by one workgroup and read by another (planes, fm) is stored with device scope, followed by a
-// wait for the acknowledgement and an arrival count; the reader passes an acquire fence after it has seen
-// the count.
-// =======================================================================================
-
-// Layout of the synchronisation words, in cache lines of SYNC_LINE ints (conv_sync_lines() of them): line 0 the XCDs
-// whose workgroups have all left, line 1 a flag (a wait that cannot time out did), lines 2.. the eight phase-0 queues,
-// then per queue the chunks of it that are written, then per XCD the workgroups that have left, then the number of
-// phase-0 queues whose chunks are all written, then two lines per column tile: finished tiles, phase-2 queue.
-constexpr int LINE_LEFT_ALL = 0, LINE_GAVE_UP = 1, LINE_Q0 = 2, LINE_DONE0 = 10, LINE_LEFT = 18, LINE_ALLDONE0 = 26,
-              LINE_SLAB0 = CONV_LINE_SLAB0;
-
-// Diagnostic build (-DSHFLBW_CONV_STAMPS): workgroups 0 and 100 leave 100 MHz timestamps of their phase boundaries
-// in the flag line of the synchronisation words (ints 16.. of line 1).
-#ifdef SHFLBW_CONV_STAMPS
-#define CONV_STAMP(i)                                                                                           \
-    do {                                                                                                        \
-        if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100))                                                 \
-            ((unsigned long long*)(c.sync + LINE_GAVE_UP * SYNC_LINE + 16))[(blockIdx.x == 0 ? 0 : 12) + (i)] = wall_clock64(); \
-    } while (0)
-#else
-#define CONV_STAMP(i) do { } while (0)
-#endif
-
-__device__ __forceinline__ int sync_load(const int* p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // 512 threads transpose 2 * nk (nk = 1, 2 or 4) 64 x 64 fp16 tiles through LDS at `lds` (8 KiB per tile):
 // `load(tile, i, j)` returns the 16-byte piece j (8 halves) of source row i of a tile; `store(tile, o, q, v)` receives
 // the halves at source rows 8q .. 8q+7 of source column o.  Threads 0..255 own tiles 0..nk-1, threads 256..511 tiles
@@ -445,200 +316,302 @@ __device__ __forceinline__ void transpose_tiles(uint32_t lds, int tid, int nk, L
     __syncthreads();
 }
 
+// =======================================================================================
+// Fused form of the convolution: ONE persistent launch in which every XCD works for itself.
+//
+// The columns of the GEMM (the padded output grid with the batch innermost, as in the batch-innermost plane form:
+// column (ho, j, img) = (ho * PW + j) * B + img, which is also the plane position tap (0, 0) of that output reads)
+// are cut into one contiguous range of `cx` columns per XCD.  The workgroups of an XCD then run three phases over
+// that range, on buffers nobody else touches and that stay in the XCD's own L2:
+//   phase 0  NHWC input -> the XCD's slab of channel-major padded planes, positions [x * cx, x * cx + cx + largest tap
+//            offset): slab[(phase * C + c) * pitch + local position]; 64 x 64 tile transposes, a few per chunk;
+//   phase 1  the role-split SpMM over the range, tiles of (row panel x column tile): the gather ids are offsets into
+//            the slab, the result rows go to the XCD's filter-major scratch fm[f][local column];
+//   phase 2  fm -> NHWC output, 64 x 64 tile transposes, padding columns (j >= Wo) dropped.
+// A phase starts when the units of work (chunks, tiles) of the one before are counted complete.  The counting is
+// between workgroups of one XCD, so it is done in that XCD's L2 (xcd_fetch_add / xcd_read, about 0.7 us a round trip
+// instead of a trip to memory), and the data handed from one workgroup to another needs no device-scope
+// write-through: it is stored normally, acknowledged by the L2 (s_waitcnt vmcnt(0)) before the writer counts it, and
+// read by compute units that have not touched those cache lines before in this launch (every line of the slab and of
+// fm has exactly one writing workgroup: tiles start at multiples of 64 values and the pitches are multiples of 64).
+//
+// Who does what is fixed, so that no unit has to be claimed (a claim is another round trip): the W = gridDim.x / nx
+// workgroups of an XCD carry the numbers l = blockIdx.x / nx = 0 .. W-1 (consecutive workgroup ids go to consecutive
+// XCDs; the host has checked that on this device), and number l does the units l, l + W, l + 2W, ... of every phase.
+// A number is taken by setting its bit in the XCD's PRESENT word.  No wait may depend on a workgroup that is not
+// running (two such launches can share the chip, each with a part of its workgroups resident): a workgroup that has
+// waited `patience` ticks for a phase looks for numbers nobody has taken, takes them and does their units as
+// well, in this and the following phases; the late owner of such a number finds its bit set and leaves at once
+// (so does a workgroup that finds itself on an XCD where its number is taken: the work is then done once, by the
+// first).  Waits are bounded all the same (`spin_ticks`): a wait that runs out raises the flag word and the
+// workgroup leaves; shflbw_spconv_check reports it.  The words are all zero between launches: the last of the W
+// workgroups of an XCD to leave clears them.
+// =======================================================================================
+
+// synchronisation words: line 0 holds the flag; XCD x owns lines 1 + x * XCD_LINES ..
+constexpr int XPRESENT = 0, XD0 = 1, XD1 = 2, XLEFT = 3;
+static_assert(XLEFT < XCD_LINES, "counter lines per XCD");
+
+// Diagnostic build (-DSHFLBW_CONV_STAMPS): workgroups 0 and 9 leave 100 MHz timestamps of their phase boundaries
+// behind the flag word (ints 16.. of line 0), and bits of `debug` switch parts of the kernel off.
+#ifdef SHFLBW_CONV_STAMPS
+#define CONV_DEBUG(bit) ((c.debug & (bit)) != 0)
+#define CONV_STAMP(i)                                                                                           \
+    do {                                                                                                        \
+        if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 9))                                                   \
+            ((unsigned long long*)(c.sync + 16))[(blockIdx.x == 0 ? 0 : 12) + (i)] = wall_clock64();            \
+    } while (0)
+#else
+#define CONV_DEBUG(bit) false
+#define CONV_STAMP(i) do { } while (0)
+#endif
+
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
-__global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_fused_kernel(SpmmLaunchArgs a, ConvFuseArgs c)
+__global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_xcd_kernel(SpmmLaunchArgs a, ConvXcdArgs c)
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
     static_assert((NCONS + NPROD) * 64 == 512 && Cfg::RING_BYTES >= 8 * TT * TT * 2, "the layout phases use 512 threads and up to 64 KiB");
     extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-    __shared__ int mailbox[2];
+    __shared__ int mailbox;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int X = a.X;
-    if (tid == 0) *(SHFLBW_LDS unsigned*)(uintptr_t)(lds0 + Cfg::LDS_BYTES) = 0u; // consumer waves count finished tiles here
-    __syncthreads();
     CONV_STAMP(0);
 
-    // ================= phase 0: NHWC input -> channel-major padded planes =================
-    if (c.phases & 1) {
-        const PlaneGeom& g = c.g;
-        const int nphase = g.stride * g.stride, PS = g.PH * g.PW;
-        // The chunk list is cut into eight ranges with a queue each; a workgroup serves the queue of its XCD first and
-        // then the others (a queue that a load shows to be exhausted is skipped without an atomic).  A chunk is written
-        // once its stores are acknowledged; the workgroup that writes the last chunk of a queue counts the queue.
-        const int per_q = (c.n0chunks + 7) >> 3;
-        const int xcd = blockIdx.x & 7;
+    const int x = xcd_id();
+    if (x >= c.nx) { // an XCD the host did not see when it probed the device: nothing here can be trusted
+        if (wave == 0) {
+            if (lane == 0) __hip_atomic_store(c.sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    int* const sx = c.sync + (1 + x * XCD_LINES) * SYNC_LINE;
+    const int W = (int)gridDim.x / c.nx;                   // workgroups of this launch on every XCD (at most 32)
+    const int me = (int)blockIdx.x / c.nx;                 // this one's number among them
+    const unsigned all_numbers = W >= 32 ? 0xffffffffu : (1u << W) - 1u;
+    const int col0 = x * c.cx;
+    const int n_x = min(c.cx, c.ncols - col0); // columns of this XCD (<= 0: none)
+
+    // Counting is done by lane 0 of wave 0.  `wave == 0` is uniform for a wave (a scalar branch: whole waves take it
+    // or skip it), and every use below is ONE such block between two workgroup barriers, so every wave passes the
+    // same barriers in the same order however the compiler arranges the lane-0 code.  (Two lane-0 blocks next to
+    // each other across a loop's back edge were merged by the compiler into a path of their own, and the other lanes
+    // of wave 0 went through the barriers of the next iteration ahead of lane 0.)
+    auto publish = [&](auto&& lane0_value) __attribute__((always_inline)) {
+        __syncthreads(); // everybody has read the previous value
+        if (wave == 0) {
+            if (lane == 0) mailbox = lane0_value();
+        }
+        __syncthreads();
+        return __builtin_amdgcn_readfirstlane(mailbox);
+    };
+
+    const PlaneGeom& g = c.g;
+    half_t* const slab = c.slabs + (size_t)x * c.slab_elems;
+    half_t* const fm = c.fm + (size_t)x * c.fm_elems;
+    SpmmLaunchArgs b = a; // the XCD's own GEMM: its slab as B, its scratch as D, local column numbers
+    b.N = max(n_x, 0);
+    b.n_tiles = (b.N + Cfg::BN - 1) / Cfg::BN;
+    b.B = slab;
+    b.D = fm;
+    b.ldd = c.cx;
+
+    // ---- units of the three phases
+    const int npos = n_x + c.max_shift; // local positions some column of this XCD reads
+    const int pos_chunks = (npos + c.pt * TT - 1) / (c.pt * TT);
+    const int n0units = n_x > 0 ? g.nwanted * c.ch_chunks * pos_chunks : 0;
+    const int n1units = n_x > 0 ? a.X * b.n_tiles : 0;
+    const int col_chunks = (n_x + c.mt * TT - 1) / (c.mt * TT);
+    const int n2units = n_x > 0 ? c.f_chunks * col_chunks : 0;
+
+    // phase 0: the chunks number l owns
+    auto phase0 = [&](int l) __attribute__((always_inline)) {
         const int nk = (c.ct * c.pt) >> 1;
-        int tried = 0;
-        while (true) {
-            if (tid == 0) {
-                int chunk = -1;
-                while (tried < 8) {
-                    const int qi = (xcd + tried) & 7;
-                    const int lo = qi * per_q, size = min(c.n0chunks, lo + per_q) - lo;
-                    int* q = c.sync + (LINE_Q0 + qi) * SYNC_LINE;
-                    if (size > 0 && sync_load(q) < size) {
-                        const int got = __hip_atomic_fetch_add(q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (got < size) {
-                            chunk = lo + got;
-                            break;
-                        }
-                    }
-                    tried++;
-                }
-                mailbox[0] = chunk;
-            }
-            __syncthreads();
-            const int chunk = __builtin_amdgcn_readfirstlane(mailbox[0]);
-            if (chunk < 0) break;
-            const int plane = chunk / (c.ch_chunks * c.pos_chunks), rem = chunk % (c.ch_chunks * c.pos_chunks);
+        int done = 0;
+        for (int chunk = l; chunk < n0units; chunk += W, done++) {
+            const int plane = chunk / (c.ch_chunks * pos_chunks), rem = chunk % (c.ch_chunks * pos_chunks);
             const int p_base = (rem / c.ch_chunks) * (c.pt * TT), c_base = (rem % c.ch_chunks) * (c.ct * TT);
-            const int copy = g.wanted[plane] / nphase, phase = g.wanted[plane] % nphase;
+            const int phase = g.wanted[plane];
             const int pa = phase / g.stride, pb = phase % g.stride;
-            half_t* dst = c.planes + ((size_t)(copy * nphase + phase) * g.C) * g.pitch;
+            half_t* dst = slab + (size_t)phase * g.C * g.pitch;
+            if (CONV_DEBUG(1)) continue;
             transpose_tiles(
                 lds0, tid, nk,
-                [&](int tile, int i, int j) { // source row = position (+ copy), piece = 8 channels
+                [&](int tile, int i, int j) { // source row = plane position, piece = 8 channels
                     half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-                    const int n = p_base + (tile / c.ct) * TT + i + copy;
+                    const int gpos = col0 + p_base + (tile / c.ct) * TT + i;
                     const int ch = c_base + (tile % c.ct) * TT + j * 8;
-                    int img, r2, prow, pcol;
-                    fast_divmod(n, PS, c.magic_ps, img, r2);
-                    fast_divmod(r2, g.PW, c.magic_pw, prow, pcol);
+                    int rem2, img, prow, pcol;
+                    fast_divmod(gpos, g.B, c.magic_b, rem2, img);
+                    fast_divmod(rem2, g.PW, c.magic_pw, prow, pcol);
                     const int hi = prow * g.stride + pa - g.pad_h, wi = pcol * g.stride + pb - g.pad_w;
-                    if (img < g.B && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && ch < g.C)
+                    if (prow < g.PH && hi >= 0 && hi < g.H && wi >= 0 && wi < g.W && ch < g.C)
                         v = *(const half8_t*)(c.in + ((size_t)(img * g.H + hi) * g.W + wi) * g.C + ch);
                     return v;
                 },
                 [&](int tile, int o, int q, half8_t v) { // destination row = channel, 8 positions
                     const int ch = c_base + (tile % c.ct) * TT + o;
                     const int p = p_base + (tile / c.ct) * TT + q * 8;
-                    if (ch < g.C && p < c.np64) store_result_16B(dst + (size_t)ch * g.pitch + p, v);
+                    if (ch < g.C && p < g.pitch) *(half8_t*)(dst + (size_t)ch * g.pitch + p) = v;
                 });
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (tid == 0) {
-                const int qi = min(chunk / per_q, 7), size = min(c.n0chunks, (qi + 1) * per_q) - qi * per_q;
-                if (__hip_atomic_fetch_add(c.sync + (LINE_DONE0 + qi) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == size - 1)
-                    __hip_atomic_fetch_add(c.sync + LINE_ALLDONE0 * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
         }
-        CONV_STAMP(1);
-        CONV_STAMP(2);
-        // Wait until every queue is written.  The planes were not read by this launch so far, so no cache holds lines of
-        // them except the up-to-date ones of their writers (caches start a launch invalidated, and the stores go through
-        // to memory): the gathers that follow need no invalidation of their own.
-        if (tid == 0) {
-            const int queues = (c.n0chunks + per_q - 1) / max(per_q, 1);
-            const unsigned long long t0 = wall_clock64();
-            while (sync_load(c.sync + LINE_ALLDONE0 * SYNC_LINE) < queues) {
-                if (wall_clock64() - t0 > 200000000ull) { // two seconds: cannot happen, chunks are only held by running workgroups
-                    __hip_atomic_store(c.sync + LINE_GAVE_UP * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(8);
-            }
-        }
-        __syncthreads();
-        CONV_STAMP(3);
-        CONV_STAMP(4);
-    }
-
-    // ================= phase 1: the SpMM over this workgroup's tiles =================
-    const int T = X * a.n_tiles;
-    const int per = (T + 7) >> 3;
-    const int S = gridDim.x >> 3;
-    const int id_first = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-    const int id_end = min(T, ((blockIdx.x & 7) + 1) * per);
-    {
+        return done;
+    };
+    // phase 1: the tiles number l owns, as one stream (the producers run ahead across its tile boundaries)
+    auto phase1 = [&](int l) __attribute__((always_inline)) {
+        if (l >= n1units || CONV_DEBUG(2)) return l < n1units ? (n1units - l + W - 1) / W : 0;
         if (wave >= NCONS)
-            ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE, true>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
+            ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE>(b, lds0, lane, wave - NCONS, l, n1units, W);
         else if constexpr (V == 16)
-            ws_consumer16<Cfg, WN, NCONS, true>(a, lds0, lane, wave, id_first, id_end, S);
+            ws_consumer16<Cfg, WN, NCONS, true>(b, lds0, lane, wave, l, n1units, W);
         else
-            ws_consumer<Cfg, V, WN, NCONS, true>(a, lds0, lane, wave, id_first, id_end, S);
-    }
-    __syncthreads(); // both roles are through: the ring is free
-    CONV_STAMP(5);
-
-    // ================= phase 2: fm[F][BN] slabs -> NHWC output =================
-    if (c.phases & 2) {
-        const int chunks_per_slab = c.f_chunks * ((Cfg::BN / TT + c.mt - 1) / c.mt);
-        const int img_cols = c.Ho * c.g.PW;
-        const unsigned long long t0 = wall_clock64();
-        // One visit to every column tile this workgroup computed a tile of (in its tile order).  A column tile that is
-        // complete is emptied; for one that is not, the workgroup waits while it has time left and moves on otherwise:
-        // the workgroup whose arrival completes it comes by later and empties it.
-        int prev = -1;
-        for (int id = id_first; id < id_end; id += S) {
-            const int s = id / X;
-            if (s == prev) continue;
-            prev = s;
-            if (tid == 0) {
-                int ok = 0;
-                while (true) {
-                    if (sync_load(c.sync + (LINE_SLAB0 + 2 * s) * SYNC_LINE) >= c.arrivals_per_slab) {
-                        ok = 1;
-                        break;
-                    }
-                    if (wall_clock64() - t0 > (unsigned long long)c.help_ticks) break;
-                    __builtin_amdgcn_s_sleep(2);
-                }
-                mailbox[1] = ok;
-            }
-            __syncthreads();
-            const int ok = __builtin_amdgcn_readfirstlane(mailbox[1]);
-            __syncthreads();
-            if (!ok) continue;
-            // the result rows were not read by this launch so far (see the planes above): no invalidation needed
-            CONV_STAMP(6);
-            CONV_STAMP(7);
-            while (true) {
-                if (tid == 0)
-                    mailbox[0] = __hip_atomic_fetch_add(c.sync + (LINE_SLAB0 + 2 * s + 1) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();
-                const int chunk = __builtin_amdgcn_readfirstlane(mailbox[0]);
-                if (chunk >= chunks_per_slab) break;
-                const int f_base = (chunk % c.f_chunks) * (c.ft * TT);
-                const int m_base = s * Cfg::BN + (chunk / c.f_chunks) * (c.mt * TT);
-                const int m_end = min(c.ncols, (s + 1) * Cfg::BN);
-                transpose_tiles(
-                    lds0, tid, (c.ft * c.mt) >> 1,
-                    [&](int tile, int i, int j) { // source row = filter, piece = 8 columns of the GEMM
-                        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-                        const int f = f_base + (tile % c.ft) * TT + i;
-                        const int m = m_base + (tile / c.ft) * TT + j * 8;
-                        if (f < c.F && m < m_end) v = *(const half8_t*)(c.fm + (size_t)f * c.ncols + m);
-                        return v;
-                    },
-                    [&](int tile, int o, int q, half8_t v) { // destination row = the pixel of column m, 8 filters
-                        const int m = m_base + (tile / c.ft) * TT + o;
-                        const int f = f_base + (tile % c.ft) * TT + q * 8;
-                        int img, r2, ho, wo;
-                        fast_divmod(m, img_cols, c.magic_imgcols, img, r2);
-                        fast_divmod(r2, c.g.PW, c.magic_pw, ho, wo);
-                        if (m < m_end && wo < c.Wo && f < c.F)
-                            *(half8_t*)(c.out + ((size_t)(img * c.Ho + ho) * c.Wo + wo) * c.F + f) = v;
-                    });
-            }
+            ws_consumer<Cfg, V, WN, NCONS, true>(b, lds0, lane, wave, l, n1units, W);
+        return (n1units - l + W - 1) / W;
+    };
+    // phase 2: the chunks number l owns
+    auto phase2 = [&](int l) __attribute__((always_inline)) {
+        for (int chunk = l; chunk < n2units; chunk += W) {
+            const int f_base = (chunk % c.f_chunks) * (c.ft * TT);
+            const int m_base = (chunk / c.f_chunks) * (c.mt * TT);
+            if (CONV_DEBUG(4)) continue;
+            transpose_tiles(
+                lds0, tid, (c.ft * c.mt) >> 1,
+                [&](int tile, int i, int j) { // source row = filter, piece = 8 columns of the GEMM
+                    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const int f = f_base + (tile % c.ft) * TT + i;
+                    const int m = m_base + (tile / c.ft) * TT + j * 8;
+                    if (f < c.F && m < n_x) v = *(const half8_t*)(fm + (size_t)f * c.cx + m);
+                    return v;
+                },
+                [&](int tile, int o, int q, half8_t v) { // destination row = the pixel of column m, 8 filters
+                    const int m = m_base + (tile / c.ft) * TT + o;
+                    const int f = f_base + (tile % c.ft) * TT + q * 8;
+                    int rem2, img, ho, wo;
+                    fast_divmod(col0 + m, g.B, c.magic_b, rem2, img);
+                    fast_divmod(rem2, g.PW, c.magic_pw, ho, wo);
+                    // streaming store: the output is not read again here
+                    if (m < n_x && wo < c.Wo && f < c.F)
+                        __builtin_nontemporal_store(v, (half8_t*)(c.out + ((size_t)(img * c.Ho + ho) * c.Wo + wo) * c.F + f));
+                });
         }
+    };
+    // Ends a phase for this workgroup: its stores are acknowledged by the L2 (every wave waits for its own before the
+    // barrier), then lane 0 counts `units` as done in `word` and waits until the word has reached `target`.  Returns
+    // -1 then; -2 when the time ran out; -3 when `refused` (this workgroup's number turned out to be somebody else's:
+    // nothing is counted); or, after `patience` ticks of waiting, a number nobody had taken and that this workgroup
+    // has taken now (its units of this phase are to be done and the phase ended again).
+    auto end_phase = [&](int* word, int units, int target, bool refused) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        return publish([&]() {
+            if (refused) return -3;
+            if (units > 0) (void)xcd_fetch_add(word, units);
+            // the clock is looked at once in 64 polls: reading it takes longer than a poll
+            unsigned long long t0 = 0, asked = 0;
+            for (unsigned polls = 1; xcd_read(word) < target; polls++) {
+                if ((polls & 63) == 0) {
+                    const unsigned long long now = wall_clock64();
+                    if (t0 == 0) t0 = asked = now;
+                    if (now - t0 > (unsigned long long)c.spin_ticks) {
+                        __hip_atomic_store(c.sync, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        return -2;
+                    }
+                    if (now - asked > (unsigned long long)c.patience) {
+                        asked = now;
+                        const unsigned missing = all_numbers & ~(unsigned)xcd_read(sx + XPRESENT * SYNC_LINE);
+                        if (missing) {
+                            const int l = __builtin_ctz(missing);
+                            if (!((unsigned)xcd_fetch_or(sx + XPRESENT * SYNC_LINE, (int)(1u << l)) & (1u << l))) return l;
+                        }
+                    }
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            return -1;
+        });
+    };
+
+    // ---- take this workgroup's number; the answer is looked at after its first units (the atomic is under way
+    // while they run: what a second holder of a number writes is what the first one writes)
+    unsigned taken_before = 0;
+    if (wave == 0) {
+        if (lane == 0) taken_before = (unsigned)xcd_fetch_or(sx + XPRESENT * SYNC_LINE, (int)(1u << me));
+    }
+    unsigned mine = 1u << me; // the numbers this workgroup does the units of
+    bool alive = n_x > 0;
+
+    // ================= phase 0: NHWC input -> this XCD's slab of planes =================
+    // (each phase: the units of the numbers in `todo`, then the end of the phase - which may come back with one more
+    // number, if one had to be taken over)
+    unsigned todo = mine;
+    for (bool first = true; alive; first = false) {
+        int units = 0;
+        for (unsigned m = todo; m; m &= m - 1) units += phase0(__builtin_ctz(m));
+        if (first) CONV_STAMP(1);
+        // While the workgroup waits for the phase: the first stages of its first tile of phase 1 (kept-column ids,
+        // A fragments) are read once by two waves that have nothing to do, so that the producers find them in the
+        // L2 instead of waiting for memory twice in a row.  The loads are issued here and looked at after the wait.
+        int w0 = 0, w1 = 0, w2 = 0;
+        if (first && me < n1units && (wave == 1 || wave == 2) && !CONV_DEBUG(32)) {
+            const int2_t pd = ((const SHFLBW_CONST int2_t*)(uintptr_t)a.panel_desc)[me % a.X];
+            const int groups = (pd.x + 3) / 4; // 64-slot groups of the panel
+            const char* src = wave == 1 ? (const char*)(KT == 16 ? a.kidx_pm : a.kidx) + (size_t)pd.y * 256
+                                        : (const char*)a.packedA + (size_t)pd.y * (64 * V * 2);
+            const size_t bytes = wave == 1 ? (size_t)min(groups, 8) * 256 : (size_t)min(groups, 3) * (64 * V * 2);
+            const size_t off = (size_t)lane * 128; // one value per 128-byte line, 8 KiB per round of the wave
+            if (off < bytes) w0 = *(const int*)(src + off);
+            if (off + 8192 < bytes) w1 = *(const int*)(src + off + 8192);
+            if (off + 16384 < bytes) w2 = *(const int*)(src + off + 16384);
+        }
+        // (a number somebody else holds already: that workgroup does, or did, its units)
+        const int r = end_phase(sx + XD0 * SYNC_LINE, units, n0units, first && ((taken_before >> me) & 1u));
+        asm volatile("" : : "v"(w0), "v"(w1), "v"(w2));
+        if (r == -1) break;
+        if (r < -1) alive = false;
+        else mine |= (todo = 1u << r);
+    }
+    CONV_STAMP(2);
+
+    // ================= phase 1: the SpMM over this XCD's columns =================
+    todo = mine;
+    for (bool first = true; alive; first = false) {
+        int units = 0;
+        for (unsigned m = todo; m; m &= m - 1) units += phase1(__builtin_ctz(m));
+        if (first) CONV_STAMP(3);
+        const int r = end_phase(sx + XD1 * SYNC_LINE, units, n1units, false); // a number without units in phase 0 may still be free
+        if (r == -1) break;
+        if (r < -1) alive = false;
+        else mine |= (todo = 1u << r);
+    }
+    CONV_STAMP(4);
+
+    // ================= phase 2: this XCD's fm[F][n_x] -> NHWC output =================
+    if (alive) {
+        for (unsigned m = mine; m; m &= m - 1) phase2(__builtin_ctz(m));
+        CONV_STAMP(5);
     }
 
-    // ================= leave: the last workgroup clears the words for the next launch =================
-    // counted per XCD first (one line each), then the XCDs on one line
+    // ================= leave: the last workgroup of the XCD clears its words for the next launch =================
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    CONV_STAMP(8);
-    if (tid == 0) {
-        const int xcd = blockIdx.x & 7, per_xcd = (int)gridDim.x >> 3; // the grid is a multiple of 8
-        if (__hip_atomic_fetch_add(c.sync + (LINE_LEFT + xcd) * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == per_xcd - 1 &&
-            __hip_atomic_fetch_add(c.sync + LINE_LEFT_ALL * SYNC_LINE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 7) {
-            for (int i = 0; i < LINE_SLAB0 + 2 * c.slabs; i++)
-                if (i != LINE_GAVE_UP) __hip_atomic_store(c.sync + i * SYNC_LINE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    CONV_STAMP(6);
+    if (wave == 0) {
+        if (lane == 0) {
+            const int before = xcd_fetch_add(sx + XLEFT * SYNC_LINE, 1);
+            if (before == W - 1)
+                for (int i = 0; i <= XLEFT; i++)
+                    __hip_atomic_store(sx + i * SYNC_LINE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            else if (before >= W) // more workgroups on this XCD than its share: the counting was wrong
+                __hip_atomic_store(c.sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+}
+
+// One wave per workgroup reports the XCD it runs on: the host checks that workgroup i of a launch lands on XCD
+// i % nx before it lets the fused form count on that.
+__global__ void xcd_probe_kernel(int* out)
+{
+    if (threadIdx.x == 0) out[blockIdx.x] = xcd_id();
 }
 
 // Kept-column ids of the packed image (k = (r*S + t)*C + c per slot) -> element offsets into the plane
@@ -691,21 +664,6 @@ hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, i
 {
     const dim3 grid((NP + TT - 1) / TT, (F + TT - 1) / TT);
     hipLaunchKernelGGL(planes_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, NP, B, PH, PW, Ho, Wo, batch_inner);
-    return hipGetLastError();
-}
-
-hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream)
-{
-    const dim3 grid(NP / TT, (a.C + TT - 1) / TT, a.R);
-    hipLaunchKernelGGL(im2col_nhwc_kernel, grid, dim3(256), 0, stream, a.in, bm, a.B, a.H, a.W, a.C, a.S, a.stride,
-                       a.pad_h, a.pad_w, a.Ho, a.Wo, NP);
-    return hipGetLastError();
-}
-
-hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int npix, int NP, hipStream_t stream)
-{
-    const dim3 grid(NP / TT, (F + TT - 1) / TT);
-    hipLaunchKernelGGL(transpose_to_nhwc_kernel, grid, dim3(256), 0, stream, dm, out, F, npix, NP);
     return hipGetLastError();
 }
 
@@ -775,7 +733,7 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_chwb_kernel(SpmmL
     const int id_first = xcd * per + (blockIdx.x >> 3);
     const int id_end = min(T, (xcd + 1) * per);
     if (wave >= NCONS)
-        ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE, false>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
+        ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
     else if constexpr (V == 16)
         ws_consumer16<Cfg, WN, NCONS, false, true>(a, lds0, lane, wave, id_first, id_end, S);
     else
@@ -827,48 +785,52 @@ const ConvChwbKernel* conv_chwb_kernel(int V)
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
-static hipError_t launch_fused(const SpmmLaunchArgs& a, const ConvFuseArgs& c, hipStream_t stream)
+static hipError_t launch_xcd(const SpmmLaunchArgs& a, const ConvXcdArgs& c, hipStream_t stream)
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
-    SpmmLaunchArgs b = a;
-    b.n_tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
-    const int T = a.X * b.n_tiles;
+    // one persistent workgroup per compute unit, the same number on every XCD
     int grid = a.num_cus > 0 ? a.num_cus : 256;
-    grid = (grid / 8) * 8;
-    const int need = ((T + 7) / 8) * 8;
-    if (grid > need) grid = need;
-    hipLaunchKernelGGL((spconv_fused_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid), dim3(Cfg::THREADS),
-                       Cfg::LDS_BYTES + 16, stream, b, c);
+    grid = (grid / c.nx) * c.nx;
+    if (grid <= 0 || c.nx <= 0 || grid / c.nx > 32 || c.cx <= 0 || (c.cx % TT) != 0 || (c.g.pitch % TT) != 0 || c.g.pitch < c.cx + c.max_shift)
+        return hipErrorInvalidValue;
+    hipLaunchKernelGGL((spconv_xcd_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>), dim3(grid), dim3(Cfg::THREADS), Cfg::LDS_BYTES,
+                       stream, a, c);
     return hipGetLastError();
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>
-static hipError_t prepare_fused()
+static hipError_t prepare_xcd()
 {
     using Cfg = SpmmWsCfg<V, WN, NCONS, NPROD, KT, NSTAGE>;
-    return hipFuncSetAttribute((const void*)spconv_fused_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES + 16);
+    return hipFuncSetAttribute((const void*)spconv_xcd_kernel<V, WN, NCONS, NPROD, KT, NSTAGE>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
 }
 
-#define SHFLBW_FUSED(V, WN, NC, NP, KT, NS)                                                                     \
-    {                                                                                                           \
-        V, WN* NC, NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS>::LDS_BYTES + 16, &launch_fused<V, WN, NC, NP, KT, NS>, \
-            &prepare_fused<V, WN, NC, NP, KT, NS>                                                               \
+#define SHFLBW_XCD(V, WN, NC, NP, KT, NS)                                                                            \
+    {                                                                                                                \
+        V, WN* NC, (NC + NP) * 64, SpmmWsCfg<V, WN, NC, NP, KT, NS>::LDS_BYTES, &launch_xcd<V, WN, NC, NP, KT, NS>,  \
+            &prepare_xcd<V, WN, NC, NP, KT, NS>                                                                      \
     }
 
 // one fused kernel per block height: the tile shape of the SpMM default of that height
-static const ConvFusedKernel g_fused[] = {
-    SHFLBW_FUSED(64, 128, 4, 4, 32, 4),
-    SHFLBW_FUSED(32, 128, 4, 4, 32, 4),
-    SHFLBW_FUSED(16, 128, 4, 4, 32, 4),
-    SHFLBW_FUSED(128, 64, 4, 4, 32, 6),
+static const ConvXcdKernel g_xcd[] = {
+    SHFLBW_XCD(64, 128, 4, 4, 32, 4),
+    SHFLBW_XCD(32, 128, 4, 4, 32, 4),
+    SHFLBW_XCD(16, 128, 4, 4, 32, 4),
+    SHFLBW_XCD(128, 64, 4, 4, 32, 6),
 };
 
-const ConvFusedKernel* conv_fused_kernel(int V)
+const ConvXcdKernel* conv_xcd_kernel(int V)
 {
-    for (const ConvFusedKernel& k : g_fused)
+    for (const ConvXcdKernel& k : g_xcd)
         if (k.V == V) return &k;
     return nullptr;
+}
+
+hipError_t launch_xcd_probe(int* out, int blocks, hipStream_t stream)
+{
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(blocks), dim3(64), 0, stream, out);
+    return hipGetLastError();
 }
 
 template <int V, int WN, int NWAVES, int KT>

@@ -43,40 +43,42 @@ struct PlaneGeom {
 
 bool fill_wanted_planes(PlaneGeom& g, int R, int S);
 
-// Arguments of the fused (single launch) form beside those of the SpMM in its middle.
-struct ConvFuseArgs {
-    PlaneGeom g;          // input side (phase 0)
+// Arguments of the fused (single launch, XCD-local) form beside those of the SpMM in its middle.  The columns of
+// the GEMM are those of the batch-innermost plane form (the padded output grid, ncols = Ho * PW * B); XCD x owns
+// columns [x * cx, (x + 1) * cx) and, for them, a slab of planes, a filter-major result and a set of counters.
+struct ConvXcdArgs {
+    PlaneGeom g;          // input side: PH = Ho + (R-1)/stride rows, PW columns, pitch = values per channel row of a slab
     const half_t* in;     // NHWC input
-    half_t* planes;
-    int np64;             // plane positions written per channel row (rounded up to 64)
-    int ct, pt;           // phase-0 chunk: ct channel tiles x pt position tiles of 64 (ct * pt = 8, 4 or 2)
-    int ch_chunks, pos_chunks, n0chunks; // chunks per plane along channels / positions, and in total
-    const half_t* fm;     // [F][ncols] filter-major result (phase 1 output, phase 2 input)
     half_t* out;          // NHWC output
-    int F, ncols, Ho, Wo;
-    int ft, mt;           // phase-2 chunk: ft filter tiles x mt column tiles of 64 (ft * mt = 8, 4 or 2)
-    int f_chunks;         // chunks per column tile along F
-    int slabs;            // column tiles of the GEMM
-    int arrivals_per_slab; // finished tiles that complete a column tile (one per row panel)
-    int* sync;            // synchronisation words, conv_sync_lines(slabs) cache lines of SYNC_LINE ints, all zero between launches
-    unsigned magic_ps, magic_pw, magic_imgcols; // udiv_magic of PH*PW, PW and Ho*PW
-    int help_ticks;       // 100 MHz ticks a workgroup without obligation keeps waiting for column tiles in phase 2
-    int phases;           // bit 0: run phase 0, bit 1: run phase 2 (cleared: the layout kernels are launched around it)
+    half_t* slabs;        // nx slabs of slab_elems values: [stride^2 * C + 1][pitch], the last row stays zero
+    size_t slab_elems;
+    half_t* fm;           // nx results of fm_elems values: [F][cx]
+    size_t fm_elems;
+    int* sync;            // conv_xcd_sync_lines(nx) cache lines of SYNC_LINE ints, all zero between launches
+    int nx, cx, ncols;    // XCDs, columns per XCD (a multiple of 64), columns in all
+    int max_shift;        // largest tap offset: columns [n, n + max_shift] of a slab row feed column n
+    int F, Ho, Wo;
+    int ct, pt, ch_chunks; // phase-0 chunk: ct channel tiles x pt position tiles of 64 (ct * pt = 8, 4 or 2); chunks along C
+    int ft, mt, f_chunks;  // phase-2 chunk: ft filter tiles x mt column tiles of 64; chunks along F
+    unsigned magic_b, magic_pw; // udiv_magic of B and PW
+    int spin_ticks;       // 100 MHz ticks a workgroup waits for a phase of its XCD to complete before it gives up
+    int patience;         // ... and before it looks for work of workgroups that have not started
+    int debug;            // diagnostic builds only: bits that switch parts of the kernel off (0 otherwise)
 };
 
-struct ConvFusedKernel {
+struct ConvXcdKernel {
     int V;
     int BN;      // columns of the GEMM per tile
-    int ncons;   // consumer waves per workgroup (arrivals per tile)
     int threads;
     int lds_bytes;
-    hipError_t (*launch)(const SpmmLaunchArgs&, const ConvFuseArgs&, hipStream_t);
+    hipError_t (*launch)(const SpmmLaunchArgs&, const ConvXcdArgs&, hipStream_t);
     hipError_t (*prepare)();
 };
-const ConvFusedKernel* conv_fused_kernel(int V);
-// cache lines of synchronisation words the fused form needs for a problem with `slabs` column tiles
-constexpr int CONV_LINE_SLAB0 = 27; // first of the two lines per column tile
-inline int conv_sync_lines(int slabs) { return CONV_LINE_SLAB0 + 2 * slabs; }
+const ConvXcdKernel* conv_xcd_kernel(int V);
+constexpr int XCD_LINES = 4; // cache lines of counters per XCD
+inline int conv_xcd_sync_lines(int nx) { return 1 + nx * XCD_LINES; }
+// writes the XCD every workgroup of a launch of `blocks` workgroups runs on to out[blocks] (device memory)
+hipError_t launch_xcd_probe(int* out, int blocks, hipStream_t stream);
 
 // Batch-innermost (C-H-W-B in, F-H-W-B out) form of the convolution: the copy into padded phase planes and the
 // role-split kernel whose epilogue writes compact output rows.
@@ -106,10 +108,5 @@ hipError_t launch_planes_to_nhwc(const half_t* dm, half_t* out, int F, int NP, i
 // row of `pitch` zeros in `planes`, which the same launch clears.
 hipError_t launch_plane_ids(const int* kidx, int* ids, int* ids_pm, int slots, int C, int S, int stride, int PW,
                             int pitch, int copies, int zero_id, half_t* planes, hipStream_t stream);
-
-// Stages 1 and 3 of the im2col form of the convolution: NHWC input -> im2col matrix with rows of NP
-// halves (NP a multiple of 64), and filter-major result -> NHWC output.
-hipError_t launch_im2col_nhwc(const SpconvLaunchArgs& a, half_t* bm, int NP, hipStream_t stream);
-hipError_t launch_transpose_to_nhwc(const half_t* dm, half_t* out, int F, int npix, int NP, hipStream_t stream);
 
 } // namespace shflbw

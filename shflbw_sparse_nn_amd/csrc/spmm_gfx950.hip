@@ -282,7 +282,7 @@ spmm_shflbw_ws_kernel(SpmmLaunchArgs a)
     const int id_end = min(T, (xcd + 1) * per);
 
     if (wave >= NCONS) {
-        ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE, false>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
+        ws_producer<Cfg, V, NCONS, NPROD, KT, NSTAGE>(a, lds0, lane, wave - NCONS, id_first, id_end, S);
         return;
     }
 

@@ -26,8 +26,6 @@ struct SpmmLaunchArgs {
     unsigned dmap_magic;      // udiv magic of dmap_row
     float alpha, beta;
     int num_cus; // compute units of the device (persistent kernels size their grid with it)
-    int img_cols, img_skip; // convolution only: column m of the GEMM is plane position m + (m / img_cols) * img_skip
-    int* tile_arrivals;     // fused convolution only: word nt * 2 * SYNC_LINE counts the finished tiles of column tile nt
     int alternate; // role-split kernels: walk every second tile of a workgroup from its last stage to its first
                    // (pays when the rows of B under one column tile do not fit the XCD's L2)
 };

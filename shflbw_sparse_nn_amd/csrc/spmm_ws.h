@@ -91,22 +91,6 @@ __device__ __forceinline__ void producer_tail()
     }
 }
 
-// A consumer wave has stored its part of a tile of column tile `nt`: once those stores (device scope, written
-// through) are acknowledged it counts itself in an LDS word, and the wave that completes the workgroup's NCONS
-// adds one to the arrival count of that column tile (one cache line per count, SYNC_LINE ints apart).  Kernels
-// that post-process whole column tiles (the fused convolution) wait for one arrival per tile.
-template <int NCONS>
-__device__ __forceinline__ void tile_done_signal(const SpmmLaunchArgs& a, int nt, int lane, uint32_t lds_word)
-{
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0) {
-        const unsigned before = __hip_atomic_fetch_add((SHFLBW_LDS unsigned*)(uintptr_t)lds_word, 1u, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (before % NCONS == NCONS - 1)
-            __hip_atomic_fetch_add(a.tile_arrivals + (size_t)nt * (2 * SYNC_LINE), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-}
-
 // Convolution over batch-innermost feature maps: the columns of the GEMM are the positions (i, j, b) of a padded
 // output grid, a.dmap_row of them per grid row, of which the first a.dmap_valid are output values.  Maps a column
 // (a multiple of 8; dmap_row and dmap_valid are multiples of 8 too) to its column in the compact output row and
@@ -157,7 +141,9 @@ struct TileWalker {
 // per-wave epilogue area; the barrier protocol is: after START_BARRIERS start-up barriers, barrier
 // number t (counted from 0) is passed once stage t of the workgroup's stage stream is complete in
 // LDS; a consumer executes one barrier before its first stage and one more per stage.
-template <typename Cfg, int V, int WN, int NCONS, bool SIGNAL = false, bool DMAP = false>
+// XCD_LOCAL: the result is read back by workgroups of the same XCD in the same launch and is stored without device
+// scope (it stays in that XCD's L2); DMAP: see output_column().
+template <typename Cfg, int V, int WN, int NCONS, bool XCD_LOCAL = false, bool DMAP = false>
 __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
                                             int id_end, int S)
 {
@@ -344,7 +330,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
                                     v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
                         }
 #pragma unroll
-                        for (int it = 0; it < NIT; it++) store_result_16B(a.D + roff[it] + col, v[it]);
+                        for (int it = 0; it < NIT; it++) store_result_16B<!XCD_LOCAL>(a.D + roff[it] + col, v[it]);
                     }
                 }
             }
@@ -367,14 +353,13 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) epi_block(mb, T{}, T{});
         }
-        if (SIGNAL) tile_done_signal<NCONS>(a, w.id / X, lane, lds0 + Cfg::LDS_BYTES);
     }
 }
 
 // Consumer role for block height 16: 16x16x32 tiles, one 32-slot step per LDS stage, same barrier
 // protocol and ring as ws_consumer.  Wave `cw` owns the 16 x WN sub-tile at column cw*WN.  A lane of
 // the result holds output row lane % 16 and, per 16-column block, the 4 columns 4*(lane/16) + 0..3.
-template <typename Cfg, int WN, int NCONS, bool SIGNAL = false, bool DMAP = false>
+template <typename Cfg, int WN, int NCONS, bool XCD_LOCAL = false, bool DMAP = false>
 __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int cw, int id_first,
                                               int id_end, int S)
 {
@@ -487,10 +472,9 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
                         for (int e = 0; e < 8; e++) v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
                 }
 #pragma unroll
-                for (int it = 0; it < 2; it++) store_result_16B(a.D + roff[it] + col, v[it]);
+                for (int it = 0; it < 2; it++) store_result_16B<!XCD_LOCAL>(a.D + roff[it] + col, v[it]);
             }
         }
-        if (SIGNAL) tile_done_signal<NCONS>(a, w.id / X, lane, lds0 + Cfg::LDS_BYTES);
     }
 }
 
@@ -529,10 +513,8 @@ __device__ __forceinline__ void gather_rows4(int4_t k, uint32_t rowbytes, const 
 }
 
 // Producer role: wave `pw` of NPROD issues its share of every stage of the workgroup's tile list (ids
-// id_first, id_first + S, ... < id_end; id = column tile * X + panel).  CONV maps the columns of the GEMM onto
-// plane positions: column m lies a.img_skip values further for every a.img_cols columns before it (the rows of
-// an image's plane that are no output rows are not columns of the GEMM).
-template <typename Cfg, int V, int NCONS, int NPROD, int KT, int NSTAGE, bool CONV>
+// id_first, id_first + S, ... < id_end; id = column tile * X + panel).
+template <typename Cfg, int V, int NCONS, int NPROD, int KT, int NSTAGE>
 __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t lds0, int lane, int pw, int id_first,
                                             int id_end, int S)
 {
@@ -613,7 +595,6 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
             const int lc = ((((pc >> 1) ^ row_xor32(key))) << 1) | (pc & 1);
             const int col = n0 + lc * 8;
             int c = col < N ? col : n0; // columns past N are never stored; any valid column of the tile will do
-            if (CONV) c += (c / a.img_cols) * a.img_skip;
             voff[j] = (uint32_t)c * 2;
         }
     };

@@ -45,19 +45,32 @@ struct shflbw_weight {
     void* d_packed_values = nullptr;
     void* d_packed_slab = nullptr;
 
-    // Device scratch of the convolution (layout-transformed input, filter-major result, the kept-column ids
-    // rewritten as plane offsets, synchronisation words): one allocation per distinct (form, geometry, input
-    // tensor, output tensor), handed out by shflbw_spconv_init under `scratch_lock` and kept until the weight
-    // is re-initialised or destroyed.  States over different tensors therefore never share scratch; two
-    // states with equal key are the same computation.
-    struct Scratch {
-        size_t bytes;
+    // Device scratch of the convolution, handed out by shflbw_spconv_init under `scratch_lock` and kept until the
+    // weight is re-initialised or destroyed (or shflbw_weight_release_scratch).  Two kinds:
+    //  * ConvIds: the kept-column ids rewritten as offsets into the layout-transformed input (slot order, then
+    //    producer-major order).  They depend on the form and the geometry only, so one copy per (form, B, H, W,
+    //    stride) serves every state; never recycled (a few hundred KB per geometry).
+    //  * ConvBulk: the layout-transformed input, the filter-major result and the synchronisation words of one
+    //    state, keyed by (form, geometry, input tensor, output tensor), so states over different tensors never
+    //    share them and may run on different streams.  At most CONV_BULK_DEPTH of them exist per weight: one more
+    //    distinct key recycles the least recently initialised one (same size: no allocation, no memset).
+    struct ConvIds {
+        int key[5]; // form, B, H, W, stride
         void* ptr;
-        int key[5]; // variant, B, H, W, stride
+        size_t bytes;
+    };
+    struct ConvBulk {
+        int key[5];
         const void* in;
         const void* out;
+        void* ptr;
+        size_t bytes;
+        unsigned long long stamp; // value of bulk_clock when it was last handed out
     };
-    std::vector<Scratch> conv_scratch;
+    static constexpr int CONV_BULK_DEPTH = SHFLBW_CONV_SCRATCH_DEPTH;
+    std::vector<ConvIds> conv_ids;
+    std::vector<ConvBulk> conv_bulk;
+    unsigned long long bulk_clock = 0;
     std::mutex scratch_lock;
 };
 

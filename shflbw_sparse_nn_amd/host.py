@@ -230,6 +230,10 @@ class SpconvBlockwiseOp:
     def __call__(self, stream=None):
         capi.check(self._lib.shflbw_spconv_exec(C.byref(self._state), stream))
 
+    def check(self):
+        """Waits for the device and raises if a launch of the fused form on this state did not run to completion."""
+        capi.check(self._lib.shflbw_spconv_check(C.byref(self._state)))
+
 
 def spmm_variants(brow):
     lib = capi.load()

@@ -143,3 +143,29 @@ def test_conv_reference_layout_equals_nhwc_at_stride_1():
     chwb = O.spconv_reference_chwb(F, R, S, C, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"],
                                    Bn, H, W, 1, np.ascontiguousarray(x.transpose(3, 1, 2, 0)))
     assert np.array_equal(chwb.transpose(3, 1, 2, 0), nhwc)
+
+
+@pytest.mark.parametrize("stride", [2, 3])
+@pytest.mark.parametrize("permute", [False, True])
+def test_conv_reference_layout_brute_force_at_larger_strides(stride, permute):
+    """The reference's bounds rule at stride > 1 (spconv/blockwise_format.h:97-128): the OUTPUT grid is H x W too, and
+    out[f, ho, wo, b] = sum w[f, r, t, c] * in[c, ho*stride - R/2 + r, wo*stride - S/2 + t, b] with every tap outside
+    H x W reading zero.  A restatement that used H / stride outputs, dropped the stride or swapped the filter extents
+    fails here (5 x 3 filter, H != W)."""
+    C, F, V, Bn, H, W, R, S = 6, 32, 16, 8, 7, 9, 5, 3
+    w = P.make_weight(F, R * S * C, V, 0.5, permute, 21, integer=True)
+    x = np.random.default_rng(22).integers(-4, 5, size=(C, H, W, Bn)).astype(np.float16)
+    A = O.densify(w).reshape(F, R, S, C).astype(np.float64)
+    y = np.zeros((F, H, W, Bn))
+    xd = x.astype(np.float64)
+    for ho in range(H):
+        for wo in range(W):
+            for r in range(R):
+                for t in range(S):
+                    hi, wi = ho * stride - R // 2 + r, wo * stride - S // 2 + t
+                    if 0 <= hi < H and 0 <= wi < W:
+                        y[:, ho, wo, :] += A[:, r, t, :] @ xd[:, hi, wi, :]
+    got = O.spconv_reference_chwb(F, R, S, C, V, 1, w["indptr"], w["indices"], w["values"], w["row_permute_ids"],
+                                  Bn, H, W, stride, x)
+    assert got.shape == (F, H, W, Bn)
+    assert np.array_equal(got, y)

@@ -19,11 +19,11 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    # 0: plane layout + SpMM + transpose, 1: one direct kernel, 2: im2col matrix + SpMM + transpose, 3: form 0 fused into
-    # one launch, 5: planes and result with the batch innermost (batches that are multiples of 8)
-    forms = (0, 3, 1, 2) if V != 16 else (0, 3, 2)
+    # 0: plane layout + SpMM + transpose, 1: one direct kernel (block heights 32, 64, 128); batches that are multiples of 8
+    # also 2: planes and result with the batch innermost, 3: the steps of 2 in one launch, every XCD on its own columns
+    forms = (0, 1) if V != 16 else (0,)
     if Bn % 8 == 0:
-        forms += (5,)
+        forms += (2, 3)
     for variant in forms:
         print("conv", (Bn, H, W, C, F, R, S, stride, V, d, permute), "form", variant, flush=True)
         got = run_spconv(torch, w, R, S, C, x, stride, variant)
@@ -48,6 +48,9 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     (24, 6, 5, 24, 48, 3, 3, 3, 16, 0.5, True),   # stride 3, block height 16, batch of 24
     (16, 4, 4, 8, 128, 1, 1, 1, 128, 0.6, True),  # 1x1 filter: no padding at all
     (8, 9, 8, 16, 64, 4, 2, 2, 32, 0.3, True),    # even filter extents: the output is larger than input / stride
+    (8, 14, 14, 24, 48, 3, 3, 1, 16, 0.3, True),  # F and C no multiples of 64: ragged tiles in the layout phases
+    (40, 9, 11, 8, 256, 3, 3, 1, 128, 0.2, True), # block height 128 (256-column tiles), batch of 40
+    (12, 28, 28, 64, 512, 3, 3, 1, 32, 0.25, True), # block height 32 with 384 <= K <= 1128 and many column tiles: the middle must stay a gather
 ])
 def test_exact_shapes(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute):
     _exact(torch_gpu, Bn, H, W, C, F, R, S, stride, V, d, permute)
@@ -92,10 +95,12 @@ def test_shift_equivariance(torch_gpu):
 
 
 def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
-    """The fused form keeps queues and arrival counts in its scratch and clears them when a launch ends: many
+    """The fused form keeps queues and counts in its scratch and clears them when a launch ends: many
     launches of one state in a row, with a new input each time, must all be right.  Two states over different
-    tensors own different scratch, so their launches may overlap on two streams."""
+    tensors own different scratch, so their launches may overlap on two streams; no wait inside depends on a
+    workgroup that is not running, so neither launch can block the other for good."""
     import shflbw_sparse_nn_amd as S
+    from shflbw_sparse_nn_amd import capi
     torch = torch_gpu
     Bn, H, W, C, F, R, Sx, stride, V = 8, 14, 14, 64, 256, 3, 3, 1, 64
     w = P.make_weight(F, R * Sx * C, V, 0.2, True, 2021, integer=True)
@@ -112,6 +117,7 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
         op.initialize(f, Bn, H, W, stride, dX[i].data_ptr(), dY[i].data_ptr())
         ops.append(op)
     assert ops[0]._state.planes != ops[1]._state.planes  # scratch is per (geometry, tensors)
+    assert ops[0]._state.spmm.packed_indices == ops[1]._state.spmm.packed_indices  # the ids per geometry only
     for rnd in range(6):
         print("fused conv round", rnd, flush=True)
         for i in range(2):
@@ -123,8 +129,66 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
                 ops[i](streams[i].cuda_stream)
         torch.cuda.synchronize()
         for i in range(2):
+            capi.check(capi.load().shflbw_spconv_check(ops[i]._state))
             np.testing.assert_array_equal(dY[i].cpu().numpy().view(np.uint16), refs[(rnd + i) % 3].view(np.uint16),
                                           err_msg="round %d stream %d" % (rnd, i))
+
+
+def test_fused_form_with_empty_row_panels(torch_gpu):
+    """Row panels that keep no vector at all (legal through shflbw_weight_set and load) have no stage: their tiles
+    are claimed, counted and written as zeros like any other."""
+    Bn, H, W, C, F, R, Sx, stride, V = 8, 6, 7, 16, 256, 3, 3, 1, 32
+    w = P.make_weight(F, R * Sx * C, V, 0.3, True, 77, integer=True)
+    X = F // V
+    keep = np.ones(X, dtype=bool)
+    keep[[0, 3, 4, X - 1]] = False  # empty panels at the start, in a row, at the end
+    counts = np.diff(w["indptr"]) * keep
+    indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    sel = np.concatenate([np.arange(w["indptr"][p], w["indptr"][p + 1]) for p in range(X) if keep[p]])
+    w2 = dict(w, nnzb=int(indptr[-1]), indptr=indptr, indices=w["indices"][sel],
+              values=w["values"].reshape(-1, V)[sel].reshape(-1))
+    x = np.random.default_rng(78).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
+    ref = O.float_to_half(P.conv_oracle(w2, R, Sx, C, x, stride))
+    for variant in (0, 2, 3):
+        got = run_spconv(torch_gpu, w2, R, Sx, C, x, stride, variant)
+        np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16), err_msg="form %d" % variant)
+
+
+def test_scratch_stays_bounded_over_fresh_tensor_pairs(torch_gpu):
+    """A serving loop whose allocator hands out new addresses initialises a state per step: the gather ids are kept
+    per geometry, the buffers the launches write are recycled, so the filter's scratch stops growing after
+    SHFLBW_CONV_SCRATCH_DEPTH tensor pairs - and every result is still right."""
+    import ctypes as C_
+    import shflbw_sparse_nn_amd as S
+    from shflbw_sparse_nn_amd import capi
+    torch = torch_gpu
+    lib = capi.load()
+    Bn, H, W, C, F, R, Sx, stride, V = 8, 10, 10, 16, 64, 3, 3, 1, 32
+    w = P.make_weight(F, R * Sx * C, V, 0.3, True, 5, integer=True)
+    f = P.upload_weight(w, R, Sx, C, cls=S.BlockwiseSpFilter)
+    x = np.random.default_rng(6).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
+    ref = O.float_to_half(P.conv_oracle(w, R, Sx, C, x, stride))
+    hx = P.to_dev(torch, x)
+    keep, sizes = [], []
+    for variant in (0, 2, 3):
+        for i in range(40):
+            dX, dY = hx.clone(), torch.full(ref.shape, float("nan"), dtype=torch.float16, device="cuda")
+            keep.append((dX, dY))  # held, so that every pair has a fresh address
+            op = S.SpconvBlockwiseOp(variant)
+            op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr())
+            op(torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+            b, n = C_.c_size_t(0), C_.c_int(0)
+            capi.check(lib.shflbw_weight_scratch_bytes(f._h, C_.byref(b), C_.byref(n)))
+            sizes.append((b.value, n.value))
+        # flat from the depth of the pool on (this form's buffers have replaced the previous form's by then)
+        assert len(set(sizes[-30:])) == 1, sizes[-30:]
+    assert sizes[-1][1] <= 3 + 4  # one set of ids per form, at most SHFLBW_CONV_SCRATCH_DEPTH bulk buffers
+    capi.check(lib.shflbw_weight_release_scratch(f._h))
+    b, n = C_.c_size_t(1), C_.c_int(1)
+    capi.check(lib.shflbw_weight_scratch_bytes(f._h, C_.byref(b), C_.byref(n)))
+    assert (b.value, n.value) == (0, 0)
 
 
 def test_non_finite_input_does_not_leak_through_padding(torch_gpu):
@@ -141,18 +205,19 @@ def test_non_finite_input_does_not_leak_through_padding(torch_gpu):
     with np.errstate(invalid="ignore", over="ignore"):
         ref = O.float_to_half(P.conv_oracle(w, R, Sx, C, x, stride))
     assert np.isfinite(ref.astype(np.float32)).any() and not np.isfinite(ref.astype(np.float32)).all()
-    for variant in (0, 1, 2, 3):
+    for variant in (0, 1):
         got = run_spconv(torch_gpu, w, R, Sx, C, x, stride, variant)
         assert np.array_equal(np.isnan(got), np.isnan(ref)), "form %d: NaN pattern differs" % variant
         ok = ~np.isnan(ref)
         np.testing.assert_array_equal(got[ok], ref[ok], err_msg="form %d" % variant)
-    # the batch-innermost form needs a batch of eights: the same two images four times over
+    # the batch-innermost forms need a batch of eights: the same two images four times over
     x8 = np.concatenate([x] * 4)
     with np.errstate(invalid="ignore", over="ignore"):
         ref8 = O.float_to_half(P.conv_oracle(w, R, Sx, C, x8, stride))
-    got = run_spconv(torch_gpu, w, R, Sx, C, x8, stride, 5)
-    assert np.array_equal(np.isnan(got), np.isnan(ref8)), "form 5: NaN pattern differs"
-    np.testing.assert_array_equal(got[~np.isnan(ref8)], ref8[~np.isnan(ref8)], err_msg="form 5")
+    for variant in (2, 3):
+        got = run_spconv(torch_gpu, w, R, Sx, C, x8, stride, variant)
+        assert np.array_equal(np.isnan(got), np.isnan(ref8)), "form %d: NaN pattern differs" % variant
+        np.testing.assert_array_equal(got[~np.isnan(ref8)], ref8[~np.isnan(ref8)], err_msg="form %d" % variant)
 
 
 @pytest.mark.parametrize("Bn,H,W,C,F,R,S,stride,V,d,permute", [
@@ -224,10 +289,20 @@ def test_reference_layout_seeded_random_shapes(torch_gpu):
         np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
 
 
-def test_batch_innermost_form_needs_a_batch_of_eights(torch_gpu):
+@pytest.mark.parametrize("variant", [2, 3])
+def test_batch_innermost_forms_need_a_batch_of_eights(torch_gpu, variant):
     from shflbw_sparse_nn_amd import capi
     w = P.make_weight(64, 9 * 8, 32, 0.3, True, 3, integer=True)
     x = np.zeros((4, 5, 5, 8), dtype=np.float16)
     with pytest.raises(capi.ShflbwError) as e:
-        run_spconv(torch_gpu, w, 3, 3, 8, x, 1, 5)
+        run_spconv(torch_gpu, w, 3, 3, 8, x, 1, variant)
     assert e.value.status == capi.ERR_SHAPE
+
+
+def test_direct_kernel_names_its_block_sizes(torch_gpu):
+    from shflbw_sparse_nn_amd import capi
+    w = P.make_weight(64, 9 * 8, 16, 0.3, True, 3, integer=True)
+    x = np.zeros((2, 5, 5, 8), dtype=np.float16)
+    with pytest.raises(capi.ShflbwError) as e:
+        run_spconv(torch_gpu, w, 3, 3, 8, x, 1, 1)
+    assert e.value.status == capi.ERR_UNSUPPORTED and "32, 64 and 128" in str(e.value)

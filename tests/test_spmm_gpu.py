@@ -114,6 +114,31 @@ def test_beta_c_epilogue(torch_gpu, permute, V):
     np.testing.assert_array_equal(got2.view(np.uint16), ref2.view(np.uint16))
 
 
+@pytest.mark.parametrize("V,M,K,N", [(16, 256, 256, 256), (32, 1024, 520, 2048), (64, 512, 384, 512), (128, 256, 256, 256)])
+def test_beta_c_epilogue_float_values(torch_gpu, V, M, K, N):
+    """With beta != 0 the library rounds twice: h = fp16(alpha * acc) goes through the staging area, then
+    D = fp16(float(h) + beta * C).  (The reference rounds the accumulator to fp16 as well, common/mma.h:336-339, and
+    then forms alpha * h + beta * C in half arithmetic, common/epilogue.h:58-62.)  The oracle rounds
+    alpha * acc + beta * C once; the two differ by at most the first rounding, half an fp16 ulp of alpha * acc
+    (2^-11 relative), plus one fp16 ulp of the result (2^-10 relative) where that moves the last rounding."""
+    w = P.make_weight(M, K, V, 0.2, True, 12, dist=("uniform", 1.0))
+    B = P.make_dense(K, N, 12, dist=("uniform", 1.0))
+    Cm = P.make_dense(M, N, 12, dist=("normal", 4.0), stream=3)
+    alpha, beta = 1.5, -0.75
+    ref = P.spmm_oracle(w, B, Cm, alpha, beta)      # fp32, one rounding to come
+    prod = P.spmm_oracle(w, B, None, alpha, 0.0)    # alpha * A * B alone
+    for variant in range(len(S.spmm_variants(V))):
+        name = S.spmm_variants(V)[variant]
+        if name.startswith("slab") and K > 1128:
+            continue
+        got = run_spmm(torch_gpu, w, B, Cmat=Cm, alpha=alpha, beta=beta, variant=variant).astype(np.float32)
+        tol = 2.0 ** -11 * np.abs(prod) + 2.0 ** -10 * np.abs(ref) + 2.0 ** -24
+        # summation order of the variant against the oracle's: a few fp32 ulps of sum |a b|, far below the above
+        tol += 2.0 ** -20 * P.abs_products_bound(w, B) * abs(alpha)
+        bad = np.abs(got - ref) > tol
+        assert not bad.any(), "%s: %d elements off by more than the two roundings allow" % (name, int(bad.sum()))
+
+
 @pytest.mark.parametrize("name", ["cfg0", "cfg1", "cfg2"])
 def test_graded_configs(torch_gpu, name):
     c = P.SPMM_CONFIGS[name]

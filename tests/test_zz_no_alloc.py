@@ -58,6 +58,21 @@ def test_static_scratch_entry_equals_init_exec(torch_gpu, V, stride):
     np.testing.assert_array_equal(y1.view(np.uint16), ref.view(np.uint16))
 
 
+def test_static_scratch_entry_block_32_mid_sized_filter(torch_gpu):
+    """Block height 32 with 384 <= R*S*C <= 1128 and many column tiles: the SpMM in the middle must be a gather variant
+    (the variant that holds the rows of B in LDS cannot walk the planes), in the static entry and in init + exec."""
+    from oracle import oracle as O
+    R = Sx = 3
+    Cc, F, V = 64, 512, 32
+    w = P.make_weight(F, R * Sx * Cc, V, 0.25, True, 2021, integer=True)
+    f = P.upload_weight(w, R, Sx, Cc, cls=S.BlockwiseSpFilter)
+    x = np.random.default_rng(19).integers(-4, 5, size=(12, 28, 28, Cc)).astype(np.float16)
+    y0, y1 = _both(torch_gpu, f, w, x, 1, R, Sx)
+    ref = O.float_to_half(P.conv_oracle(w, R, Sx, Cc, x, 1))
+    np.testing.assert_array_equal(y0.view(np.uint16), ref.view(np.uint16))
+    np.testing.assert_array_equal(y1.view(np.uint16), ref.view(np.uint16))
+
+
 def test_static_scratch_entry_refuses_what_does_not_fit(torch_gpu):
     torch = torch_gpu
     lib = capi.load()

@@ -133,6 +133,7 @@ def run_spconv(torch, w, R, Sx, Cc, x_nhwc, stride, variant=-1):
     assert op.output_hw == (Ho, Wo)
     op(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
+    op.check()
     return dY.cpu().numpy()
 
 
