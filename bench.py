@@ -14,8 +14,10 @@ for the SpMM configs, the whole convolution (every launch of the form the librar
 configuration first passes a correctness gate (bit-exact against the CPU oracle on the integer twin of the
 workload).  Timing follows the reference's benchmark (benchmark/benchmark.spmm.cu:29-50, benchmark.spconv.cu:29-50):
 W warm-up launches, then K back-to-back launches between two events on the launch stream - here WINDOWS such
-windows in a row; `ms_per_step` is the median window, the fastest and slowest are reported beside it (a single
-window of a few launches falls into the clock ramp of an idle GPU).  The line carries the roofline of the kernel and
+windows in a row; `ms_per_step` is the median window, the fastest and slowest are reported beside it.  A single
+window of a few launches falls into the clock ramp of an idle GPU (the first ~10 ms of a burst run 8-10 % slower), so
+SETTLE_MS of untimed launches go in front of the warm-up; the reference's own loop from an idle GPU is reported
+beside it (`reference_timing_loop`).  The line carries the roofline of the kernel and
 the CPU oracle timed on the host cores as a baseline (headline only); the headline also carries a dense fp16 GEMM of
 the same shape.
 """
@@ -33,6 +35,7 @@ if ROOT not in sys.path:
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix-core peak
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 WINDOWS = 5                    # timed windows of `steps` launches each; the median is the figure
+SETTLE_MS = 20.0               # untimed launches in front of the warm-up until the shader clock has settled
 
 
 def measured_traffic(config, kernel):
@@ -74,6 +77,13 @@ def timed_windows(torch, stream, op, steps, warmup, windows=WINDOWS):
     """`warmup` untimed launches, then `windows` windows of `steps` launches each, every window between its own pair
     of events, all back to back on the stream.  Returns the per-launch milliseconds of every window and the wall
     time of the timed part."""
+    # an idle GPU needs about 10 ms of load before its clock settles (the first launches of a burst run 8-10 % slower):
+    # SETTLE_MS of untimed launches first, whatever `warmup` is
+    t_end = time.time() + SETTLE_MS * 1e-3
+    while time.time() < t_end:
+        for _ in range(50):
+            op(stream.cuda_stream)
+        torch.cuda.synchronize()
     for _ in range(warmup):
         op(stream.cuda_stream)
     torch.cuda.synchronize()
@@ -134,8 +144,9 @@ def cpu_baseline(run_all, run_one, eff_flops, sub_flops, what_all, what_one, thr
 
 
 def timing_note(args):
-    return ("%d warm-up launches, then %d windows of %d back-to-back launches, each between two events on the launch "
-            "stream, operands resident; ms_per_step = median window" % (args.warmup, WINDOWS, args.steps))
+    return ("%g ms of untimed launches (clock settling) + %d warm-up launches, then %d windows of %d back-to-back launches, "
+            "each between two events on the launch stream, operands resident; ms_per_step = median window"
+            % (SETTLE_MS, args.warmup, WINDOWS, args.steps))
 
 
 def main():

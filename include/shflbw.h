@@ -142,6 +142,10 @@ int shflbw_weight_device_ref(const shflbw_weight* w, shflbw_device_ref* ref);
  * Preconditions: weight synced; bcol == 1; N % 8 == 0; B, C, D 16-byte aligned.
  * The state is a copyable POD holding raw pointers; it dangles if the weight is
  * re-initialised or destroyed (same as the reference).
+ * Rounding: fp32 accumulation; with beta == 0 one rounding to fp16 (of alpha * acc).  With beta != 0 two: alpha * acc is
+ * rounded to fp16 first, then fp16(float(that) + beta * C) - the reference rounds the accumulator to fp16 as well
+ * (common/mma.h:336-339) and then combines in half arithmetic (common/epilogue.h:58-62); a host reference that rounds
+ * alpha * acc + beta * C once differs by at most half an fp16 ulp of alpha * acc plus one ulp of the result.
  * ------------------------------------------------------------------------- */
 typedef struct shflbw_spmm_state {
     size_t shared_mem_size;

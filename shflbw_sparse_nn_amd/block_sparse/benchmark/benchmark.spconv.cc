@@ -26,6 +26,8 @@ static float run_entry(SpconvBlockwiseInitFn_t init_fn, SpconvBlockwiseExecFn_t 
         std::cerr << "operator set-up failed for this tile name" << std::endl;
         return -1.f;
     }
+    // which form of the convolution stands behind the tile name on this problem (stderr: the result line on stdout stays the reference's)
+    std::cerr << "native kernel: " << shflbw_spconv_variant_name(state.native.variant) << std::endl;
     return launch_timing::mean_launch_ms([&] { (*exec_fn)(state, stream); }, stream, /* warmup */ 10, /* repeat */ 100);
 }
 

@@ -26,6 +26,8 @@ static float run_entry(SpmmBlockwiseInitFn_t init_fn, SpmmBlockwiseExecFn_t exec
         std::cerr << "operator set-up failed for this tile name" << std::endl;
         return -1.f;
     }
+    // which native kernel stands behind the tile name on this problem (stderr: the result line on stdout stays the reference's)
+    std::cerr << "native kernel: " << shflbw_spmm_variant_name(state.native.brow, state.native.variant) << std::endl;
     return launch_timing::mean_launch_ms([&] { (*exec_fn)(state, stream); }, stream, /* warmup */ 10, /* repeat */ 100);
 }
 
