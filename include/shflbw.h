@@ -255,6 +255,10 @@ typedef struct shflbw_spconv_state {
     int plane_rows, plane_cols, plane_pitch, plane_copies;
     int ncols;
     int xcds, cols_per_xcd;
+    int patience_ticks; /* fused form: 100 MHz ticks a workgroup waits for a phase before it takes over the work of workgroups
+                         * of the launch that have not started yet (init sets 5000 = 50 us; a caller may change it).
+                         * A negative value -t is for tests of that path: a patience of one tick, and every second
+                         * workgroup joins min(t, 10000) ticks late.  The int at byte 60 of `sync` counts the take-overs. */
     void* sync;
     shflbw_spmm_state spmm;
 } shflbw_spconv_state;

@@ -876,6 +876,7 @@ int init_fused(shflbw_spconv_state* state, const shflbw_weight* f, int B, int H,
     state->ncols = (int)g.g.ncols;
     state->xcds = nx;
     state->cols_per_xcd = (int)g.cx;
+    state->patience_ticks = 5000; // 50 us
     // the SpMM in the middle, as one XCD sees it: cx columns, its slab as B, its result as D
     rc = bind_middle(state, f, g.cx, state->planes, state->result_fm, ids, ids_pm, (g.g.rows + 1) * pitch);
     if (rc != SHFLBW_OK) return rc;
@@ -1029,7 +1030,8 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
         c.magic_b = udiv_magic(a.B);
         c.magic_pw = udiv_magic(state->plane_cols);
         c.spin_ticks = 20000000; // 0.2 s
-        c.patience = 5000;       // 50 us
+        c.patience = state->patience_ticks > 0 ? state->patience_ticks : state->patience_ticks < 0 ? 1 : 5000;
+        c.late_ticks = state->patience_ticks < 0 ? std::min(-state->patience_ticks, 10000) : 0;
         c.debug = 0;
 #ifdef SHFLBW_CONV_STAMPS
         if (const char* dbg = getenv("SHFLBW_CONV_DEBUG")) c.debug = atoi(dbg);

@@ -348,7 +348,8 @@ __device__ __forceinline__ void transpose_tiles(uint32_t lds, int tid, int nk, L
 // workgroups of an XCD to leave clears them.
 // =======================================================================================
 
-// synchronisation words: line 0 holds the flag; XCD x owns lines 1 + x * XCD_LINES ..
+// synchronisation words: line 0 holds the flag and, at int XCD_TAKEOVERS, the count of take-overs since the scratch
+// was made; XCD x owns lines 1 + x * XCD_LINES ..
 constexpr int XPRESENT = 0, XD0 = 1, XD1 = 2, XLEFT = 3;
 static_assert(XLEFT < XCD_LINES, "counter lines per XCD");
 
@@ -506,10 +507,12 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_xcd_kernel(SpmmLa
         return publish([&]() {
             if (refused) return -3;
             if (units > 0) (void)xcd_fetch_add(word, units);
-            // the clock is looked at once in 64 polls: reading it takes longer than a poll
+            // the clock is looked at once in 64 polls: reading it takes longer than a poll (at every poll when the
+            // caller has set a patience below 64 ticks, which is how the tests reach the take-over path)
+            const unsigned sparse_clock = c.patience < 64 ? 0u : 63u;
             unsigned long long t0 = 0, asked = 0;
             for (unsigned polls = 1; xcd_read(word) < target; polls++) {
-                if ((polls & 63) == 0) {
+                if ((polls & sparse_clock) == 0) {
                     const unsigned long long now = wall_clock64();
                     if (t0 == 0) t0 = asked = now;
                     if (now - t0 > (unsigned long long)c.spin_ticks) {
@@ -521,7 +524,10 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_xcd_kernel(SpmmLa
                         const unsigned missing = all_numbers & ~(unsigned)xcd_read(sx + XPRESENT * SYNC_LINE);
                         if (missing) {
                             const int l = __builtin_ctz(missing);
-                            if (!((unsigned)xcd_fetch_or(sx + XPRESENT * SYNC_LINE, (int)(1u << l)) & (1u << l))) return l;
+                            if (!((unsigned)xcd_fetch_or(sx + XPRESENT * SYNC_LINE, (int)(1u << l)) & (1u << l))) {
+                                (void)__hip_atomic_fetch_add(c.sync + XCD_TAKEOVERS, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                return l;
+                            }
                         }
                     }
                 }
@@ -534,6 +540,10 @@ __global__ void __launch_bounds__((NCONS + NPROD) * 64) spconv_xcd_kernel(SpmmLa
     // ---- take this workgroup's number; the answer is looked at after its first units (the atomic is under way
     // while they run: what a second holder of a number writes is what the first one writes)
     unsigned taken_before = 0;
+    if (c.late_ticks > 0 && (me & 1)) { // tests of the take-over path: every second workgroup joins late
+        const unsigned long long t = wall_clock64();
+        while (wall_clock64() - t < (unsigned long long)c.late_ticks) __builtin_amdgcn_s_sleep(8);
+    }
     if (wave == 0) {
         if (lane == 0) taken_before = (unsigned)xcd_fetch_or(sx + XPRESENT * SYNC_LINE, (int)(1u << me));
     }

@@ -63,6 +63,7 @@ struct ConvXcdArgs {
     unsigned magic_b, magic_pw; // udiv_magic of B and PW
     int spin_ticks;       // 100 MHz ticks a workgroup waits for a phase of its XCD to complete before it gives up
     int patience;         // ... and before it looks for work of workgroups that have not started
+    int late_ticks;       // > 0 (tests only): the workgroups with odd numbers join this many ticks late
     int debug;            // diagnostic builds only: bits that switch parts of the kernel off (0 otherwise)
 };
 
@@ -75,7 +76,8 @@ struct ConvXcdKernel {
     hipError_t (*prepare)();
 };
 const ConvXcdKernel* conv_xcd_kernel(int V);
-constexpr int XCD_LINES = 4; // cache lines of counters per XCD
+constexpr int XCD_LINES = 4;      // cache lines of counters per XCD
+constexpr int XCD_TAKEOVERS = 15; // int of the first line (the one with the flag) that counts the take-overs
 inline int conv_xcd_sync_lines(int nx) { return 1 + nx * XCD_LINES; }
 // writes the XCD every workgroup of a launch of `blocks` workgroups runs on to out[blocks] (device memory)
 hipError_t launch_xcd_probe(int* out, int blocks, hipStream_t stream);

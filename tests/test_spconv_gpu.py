@@ -94,11 +94,14 @@ def test_shift_equivariance(torch_gpu):
         np.testing.assert_array_equal(got[..., w["row_permute_ids"][r]], shifted * float(w["values"][r]))
 
 
-def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
+@pytest.mark.parametrize("patience", [0, -3000])
+def test_fused_form_repeated_launches_and_two_streams(torch_gpu, patience):
     """The fused form keeps queues and counts in its scratch and clears them when a launch ends: many
     launches of one state in a row, with a new input each time, must all be right.  Two states over different
     tensors own different scratch, so their launches may overlap on two streams; no wait inside depends on a
-    workgroup that is not running, so neither launch can block the other for good."""
+    workgroup that is not running, so neither launch can block the other for good.  A negative patience makes
+    every second workgroup join 30 us late and the others take its work over after one tick of waiting: the late ones
+    find their numbers taken and leave, and the results must not change (the scratch counts the take-overs)."""
     import shflbw_sparse_nn_amd as S
     from shflbw_sparse_nn_amd import capi
     torch = torch_gpu
@@ -115,6 +118,9 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
     for i in range(2):
         op = S.SpconvBlockwiseOp(3)
         op.initialize(f, Bn, H, W, stride, dX[i].data_ptr(), dY[i].data_ptr())
+        assert op._state.patience_ticks == 5000
+        if patience:
+            op._state.patience_ticks = patience
         ops.append(op)
     assert ops[0]._state.planes != ops[1]._state.planes  # scratch is per (geometry, tensors)
     assert ops[0]._state.spmm.packed_indices == ops[1]._state.spmm.packed_indices  # the ids per geometry only
@@ -132,6 +138,12 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu):
             capi.check(capi.load().shflbw_spconv_check(ops[i]._state))
             np.testing.assert_array_equal(dY[i].cpu().numpy().view(np.uint16), refs[(rnd + i) % 3].view(np.uint16),
                                           err_msg="round %d stream %d" % (rnd, i))
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    for op in ops:  # the int at byte 60 of the synchronisation words counts the take-overs
+        words = (ctypes.c_int * 16)()
+        assert hip.hipMemcpy(words, ctypes.c_void_p(op._state.sync), 64, 2) == 0  # device to host
+        assert (words[15] > 0) == (patience < 0), words[15]
 
 
 def test_fused_form_with_empty_row_panels(torch_gpu):
