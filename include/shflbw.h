@@ -202,7 +202,8 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  * SHFLBW_CONV_SCRATCH_DEPTH such buffers exist per filter: initialising a state over one more tensor pair recycles
  * the buffers of the least recently initialised one (no allocation, no copy when the geometry is the same), whose
  * state must not be executed afterwards.  exec only launches, in order on `stream`.
- * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice):
+ * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice - variant 2 when B % 8 == 0
+ * and there are at least 2048 output pixels B*Ho*Wo, else variant 0):
  *   variant 0 = plane form, three launches: the input is rewritten once per call as channel-major padded
  *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
  *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,

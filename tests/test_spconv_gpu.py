@@ -318,3 +318,18 @@ def test_direct_kernel_names_its_block_sizes(torch_gpu):
     with pytest.raises(capi.ShflbwError) as e:
         run_spconv(torch_gpu, w, 3, 3, 8, x, 1, 1)
     assert e.value.status == capi.ERR_UNSUPPORTED and "32, 64 and 128" in str(e.value)
+
+
+@pytest.mark.parametrize("Bn,H,expected", [(8, 8, 0), (8, 16, 2), (12, 16, 0), (32, 8, 2)])
+def test_the_library_picks_the_batch_innermost_form_for_large_batches_of_eights(torch_gpu, Bn, H, expected):
+    """shflbw_spconv_init: form 2 needs a batch that is a multiple of 8 and pays from 2048 output pixels on."""
+    import shflbw_sparse_nn_amd as S
+    torch = torch_gpu
+    C, F = 8, 32
+    w = P.make_weight(F, 9 * C, 32, 0.5, True, 3, integer=True)
+    f = P.upload_weight(w, 3, 3, C, cls=S.BlockwiseSpFilter)
+    dX = torch.zeros((Bn, H, H, C), dtype=torch.float16, device="cuda")
+    dY = torch.zeros((Bn, H, H, F), dtype=torch.float16, device="cuda")
+    op = S.SpconvBlockwiseOp()
+    st = op.initialize(f, Bn, H, H, 1, dX.data_ptr(), dY.data_ptr())
+    assert st.variant == expected, (Bn * H * H, st.variant)
