@@ -143,7 +143,8 @@ def test_fused_form_repeated_launches_and_two_streams(torch_gpu, patience):
     for op in ops:  # the int at byte 60 of the synchronisation words counts the take-overs
         words = (ctypes.c_int * 16)()
         assert hip.hipMemcpy(words, ctypes.c_void_p(op._state.sync), 64, 2) == 0  # device to host
-        assert (words[15] > 0) == (patience < 0), words[15]
+        if patience < 0:  # (with the default patience a take-over is rare but legal: nothing is asserted about it)
+            assert words[15] > 0, words[15]
 
 
 def test_fused_form_with_empty_row_panels(torch_gpu):
