@@ -128,7 +128,8 @@ static bool spmm_variant_offsets32(const SpmmVariant* v) { return v && v->name[0
 // Tile choice when the caller does not force one: the table lists the preferred (persistent, 512 columns
 // wide) variant of every block size first.  When its tiles would occupy at most half of the compute units,
 // the role-split variant with 256-column tiles is taken instead (twice the tiles; measured 15-25 % faster
-// there, 5-20 % slower once the wide tiles fill the chip).
+// there, 5-20 % slower once the wide tiles fill the chip), and the one with 128-column tiles while even those
+// are no more than the compute units.
 // Block height 32 and at most SLAB_MAX_K columns: the slab variant moves less data between the L2 and the
 // compute units once a workgroup runs enough kept vectors over the 128 KiB slab it has to load first.  Taken
 // when (34 shapes measured with both kernels, each pair on one box)
@@ -160,18 +161,28 @@ static int auto_spmm_variant(const shflbw_weight* w, int N, bool allow_slab)
             seen++;
         }
     }
+    // the role-split variant of this block size with tiles of `bn` columns, -1 when there is none
+    auto role_split_with = [&](int bn) {
+        int seen = 0;
+        for (int i = 0; i < count; i++) {
+            if (all[i].V != brow) continue;
+            if (all[i].name[0] == 'w' && all[i].BN == bn) return seen; // "ws..." names
+            seen++;
+        }
+        return -1;
+    };
+    // small problems: 128-column tiles while they do not outnumber the compute units (39 shapes of block heights 32, 64
+    // and 128 measured against the wider tiles: 6-17 % faster up to one tile per compute unit, 10-25 % slower from two on)
+    if ((long)X * ((N + 127) / 128) <= device_compute_units()) {
+        const int narrow = role_split_with(128);
+        if (narrow >= 0) return narrow;
+    }
     const SpmmVariant* first = find_spmm_variant(brow, 0, nullptr);
     if (!first || first->BN != 512) return 0;
     const long wide_tiles = (long)X * ((N + 511) / 512);
     if (wide_tiles > device_compute_units() / 2) return 0;
-    int seen = 0;
-    for (int i = 0; i < count; i++) {
-        if (all[i].V != brow) continue;
-        const bool role_split = all[i].name[0] == 'w'; // "ws..." names
-        if (role_split && all[i].BN == 256) return seen;
-        seen++;
-    }
-    return 0;
+    const int medium = role_split_with(256);
+    return medium >= 0 ? medium : 0;
 }
 
 // Geometry of the plane form of a convolution and the layout of its device scratch.

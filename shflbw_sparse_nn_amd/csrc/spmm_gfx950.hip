@@ -405,6 +405,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(64, 128, 4, 16, 3),
     SHFLBW_VARIANT(64, 64, 2, 32, 3),
     SHFLBW_VARIANT(64, 32, 4, 32, 3),
+    SHFLBW_WS_VARIANT(64, 32, 4, 4, 32, 6), // 128-column tiles: problems too small for the wider ones
     // block 32
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 32, 4),
     SHFLBW_WS_VARIANT(32, 128, 4, 4, 16, 6),
@@ -415,6 +416,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_VARIANT(32, 128, 4, 16, 3),
     SHFLBW_VARIANT(32, 64, 2, 32, 3),
     SHFLBW_SLAB_VARIANT(), // weights of at most SLAB_MAX_K columns
+    SHFLBW_WS_VARIANT(32, 32, 4, 4, 32, 6), // 128-column tiles: problems too small for the wider ones
     // block 16
     SHFLBW_WS_VARIANT(16, 128, 4, 4, 32, 4),
     // block 128
@@ -422,6 +424,7 @@ static const SpmmVariant g_variants[] = {
     SHFLBW_WS_VARIANT(128, 64, 4, 4, 32, 5),
     SHFLBW_VARIANT(128, 64, 4, 32, 3),
     SHFLBW_VARIANT(128, 32, 4, 32, 3),
+    SHFLBW_WS_VARIANT(128, 32, 4, 4, 32, 6), // 128-column tiles: problems too small for the wider ones
 };
 
 // The row of zeros the padding slots gather.  `g_zero_row` is the host-side handle of the symbol; kernels get

@@ -45,7 +45,7 @@ struct SpmmWsCfg {
     static constexpr int A_FRAGS = V == 16 ? KT / 32 : KSPS * MB;
     static constexpr int STAGE_BYTES = B_BYTES + A_FRAGS * 1024;
     static constexpr int RPW = KT / NPROD;                // gathered rows per producer and stage
-    static constexpr int RPI = 1024 / ROWB;               // rows one 1 KiB copy instruction covers (BN = 256: two)
+    static constexpr int RPI = 1024 / ROWB;               // rows one 1 KiB copy instruction covers (BN = 256: two, BN = 128: four)
     static constexpr int CPW = RPW / RPI;                 // copies of B rows per producer and stage
     static constexpr int A_HI = A_FRAGS % NPROD;          // producers [0, A_HI) copy one more A fragment
     static constexpr int A_LO = A_FRAGS / NPROD;
@@ -60,7 +60,7 @@ struct SpmmWsCfg {
     // the file: at most 128 per wave) let one workgroup's epilogue stores run beside the other's stage loop.
     static constexpr int WGS_PER_CU = LDS_BYTES <= 79 * 1024 && THREADS <= 512 ? 2 : 1;
     static_assert((V % 32 == 0 || (V == 16 && KT == 32)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
-    static_assert(BN == 512 || (BN == 256 && RPW == 8), "a 1 KiB copy instruction covers one gathered row, or two");
+    static_assert(BN == 512 || ((BN == 256 || BN == 128) && RPW == 8), "a 1 KiB copy instruction covers one gathered row, two or four");
     static_assert((KT == 16 || KT == 32) && (RPW == 4 || RPW == 8), "a 64-slot group is 4 or 2 stages; rows go in fours");
     static_assert(A_LO <= 2 && (A_LO == 0 || A_HI == 0), "the same number of A fragments for all producers that copy any");
     // A producer passes one barrier before every stage it issues.  The barrier in front of stage j is the
@@ -589,9 +589,10 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             // one copy = one row of 64 pieces (swizzle key j % 4), or the rows 2j and 2j + 1 of this
-            // producer, 32 pieces each, in the lower and the upper half of the wave
-            const int key = Cfg::RPI == 1 ? j : (2 * j + (lane >> 5)) & 3;
-            const int pc = Cfg::RPI == 1 ? lane : lane & 31;
+            // producer, 32 pieces each, in the lower and the upper half of the wave, or the rows 4j .. 4j + 3,
+            // 16 pieces each, in the four quarters of the wave
+            const int key = Cfg::RPI == 1 ? j : Cfg::RPI == 2 ? (2 * j + (lane >> 5)) & 3 : lane >> 4;
+            const int pc = Cfg::RPI == 1 ? lane : Cfg::RPI == 2 ? lane & 31 : lane & 15;
             const int lc = ((((pc >> 1) ^ row_xor32(key))) << 1) | (pc & 1);
             const int col = n0 + lc * 8;
             int c = col < N ? col : n0; // columns past N are never stored; any valid column of the tile will do
@@ -636,7 +637,7 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
                         row(std::integral_constant<int, 6>{});
                         row(std::integral_constant<int, 7>{});
                     }
-                } else {
+                } else if (Cfg::RPI == 2) {
                     const bool hi = lane >= 32;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
@@ -644,10 +645,25 @@ __device__ __forceinline__ void ws_producer(const SpmmLaunchArgs& a, uint32_t ld
                         const char* src = k < 0 ? zb : (const char*)a.B + (size_t)((uint32_t)k * rowbytes);
                         global_to_lds_16B(src + voff[j], sbp + j * 0x400);
                     }
+                } else {
+                    const int q = lane >> 4; // the quarter of the wave: row 4j + q of the producer
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const int k = q == 0 ? ks[4 * j] : q == 1 ? ks[4 * j + 1] : q == 2 ? ks[4 * j + 2] : ks[4 * j + 3];
+                        const char* src = k < 0 ? zb : (const char*)a.B + (size_t)((uint32_t)k * rowbytes);
+                        global_to_lds_16B(src + voff[j], sbp + j * 0x400);
+                    }
                 }
             } else if (Cfg::RPI == 1) {
                 gather_rows4<0>(ka, rowbytes, voff, a.B, sbp);
                 if (RPW == 8) gather_rows4<4>(kb, rowbytes, voff, a.B, sbp);
+            } else if (Cfg::RPI == 4) {
+                // 256-byte rows: quarter q of the wave fetches row 4j + q
+                const int q = lane >> 4;
+                const int k0 = q == 0 ? ka.x : q == 1 ? ka.y : q == 2 ? ka.z : ka.w;
+                const int k1 = q == 0 ? kb.x : q == 1 ? kb.y : q == 2 ? kb.z : kb.w;
+                global_to_lds_16B_sbase<0x000>(a.B, (uint32_t)k0 * rowbytes + voff[0], sbp);
+                global_to_lds_16B_sbase<0x400>(a.B, (uint32_t)k1 * rowbytes + voff[1], sbp);
             } else {
                 // 512-byte rows: the lower half of the wave fetches row 2j, the upper half row 2j + 1
                 const bool hi = lane >= 32;
