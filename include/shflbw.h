@@ -202,8 +202,8 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  * SHFLBW_CONV_SCRATCH_DEPTH such buffers exist per filter: initialising a state over one more tensor pair recycles
  * the buffers of the least recently initialised one (no allocation, no copy when the geometry is the same), whose
  * state must not be executed afterwards.  exec only launches, in order on `stream`.
- * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice - variant 2 when B % 8 == 0
- * and there are at least 2048 output pixels B*Ho*Wo, else variant 0):
+ * shflbw_spconv_init_variant (variant < 0, and shflbw_spconv_init: the library's choice - variant 2 when B % 8 == 0,
+ * else variant 0):
  *   variant 0 = plane form, three launches: the input is rewritten once per call as channel-major padded
  *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
  *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,
@@ -255,6 +255,7 @@ typedef struct shflbw_spconv_state {
     void* planes;
     int plane_rows, plane_cols, plane_pitch, plane_copies;
     int ncols;
+    int middle_tile_cols; /* variants 2 and 4: columns of a tile of the SpMM launch in the middle (512, 256 or 128, by the size of the GEMM) */
     int xcds, cols_per_xcd;
     int patience_ticks; /* fused form: 100 MHz ticks a workgroup waits for a phase before it takes over the work of workgroups
                          * of the launch that have not started yet (init sets 5000 = 50 us; a caller may change it).

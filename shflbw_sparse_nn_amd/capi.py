@@ -75,7 +75,7 @@ class SpconvState(C.Structure):
                 ("packed_values", C.c_void_p), ("packed_indices", C.c_void_p), ("panel_ptr", C.c_void_p),
                 ("brow", C.c_int), ("result_fm", C.c_void_p), ("np", C.c_int),
                 ("planes", C.c_void_p), ("plane_rows", C.c_int), ("plane_cols", C.c_int), ("plane_pitch", C.c_int),
-                ("plane_copies", C.c_int), ("ncols", C.c_int), ("xcds", C.c_int), ("cols_per_xcd", C.c_int), ("patience_ticks", C.c_int),
+                ("plane_copies", C.c_int), ("ncols", C.c_int), ("middle_tile_cols", C.c_int), ("xcds", C.c_int), ("cols_per_xcd", C.c_int), ("patience_ticks", C.c_int),
                 ("sync", C.c_void_p), ("spmm", SpmmState)]
 
 

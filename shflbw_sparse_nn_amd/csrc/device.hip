@@ -752,18 +752,20 @@ int init_batch_planes(shflbw_spconv_state* state, const shflbw_weight* f, int B,
         set_error("spconv_init: the batch must be a multiple of 8 for this form (got %d)", B);
         return SHFLBW_ERR_SHAPE;
     }
-    const ConvChwbKernel* k = conv_chwb_kernel(f->brow);
-    if (!k) {
-        set_error("spconv_init: no kernel for block size %d", f->brow);
-        return SHFLBW_ERR_UNSUPPORTED;
-    }
-    SHFLBW_HIP_TRY(k->prepare());
     if (variant == FORM_CHWB) { // H and W are the extents of the output grid and the bounds of the input (spconv/blockwise_format.h:111-115)
         state->Ho = H;
         state->Wo = W;
     }
     BatchPlanes g;
     batch_planes_geometry(f, B, stride, state->Ho, state->Wo, &g);
+    // the SpMM in the middle: tile width by the size of the GEMM, as for the SpMM proper
+    const ConvChwbKernel* k = conv_chwb_kernel(f->brow, 0, f->nrow / f->brow, g.ncols, device_compute_units());
+    if (!k) {
+        set_error("spconv_init: no kernel for block size %d", f->brow);
+        return SHFLBW_ERR_UNSUPPORTED;
+    }
+    SHFLBW_HIP_TRY(k->prepare());
+    state->middle_tile_cols = k->BN;
     const int s = stride, C = f->C, S = f->S;
     const long pitch = (g.np + g.max_shift + 8 + 63) / 64 * 64;
     if (g.ncols > 0x7fffffffL || (unsigned long long)(g.rows + 1) * (unsigned long long)pitch * 2ull > 0xffffffffull) {
@@ -958,14 +960,14 @@ int shflbw_spconv_init_variant(shflbw_spconv_state* state, const shflbw_weight* 
         set_error("spconv_init: form 4 works on C-H-W-B / F-H-W-B tensors; call shflbw_spconv_init_chwb");
         return SHFLBW_ERR_INVALID;
     }
-    // the library's choice: the batch-innermost form where the batch allows it and the problem is large enough for its
-    // smaller traffic to show (one copy of the planes instead of two, no dead plane rows in the result; measured: ahead
-    // from about 3000 output pixels on, behind by 1 us at 1600), else the plane form
+    // the library's choice: the batch-innermost form wherever the batch allows it (one copy of the planes instead of
+    // two, no dead plane rows in the result; with the tile width of its SpMM chosen by the size of the GEMM it is level
+    // with the plane form on the smallest layers and ahead from a few hundred output pixels on), else the plane form
     if (variant < 0) {
         variant = FORM_PLANES;
         if (f && f->R > 0 && B > 0 && B % 8 == 0 && H > 0 && W > 0 && stride > 0) {
             const long Ho = (H + 2 * (f->R / 2) - f->R) / stride + 1, Wo = (W + 2 * (f->S / 2) - f->S) / stride + 1;
-            if (Ho > 0 && Wo > 0 && (long)B * Ho * Wo >= 2048) variant = FORM_BPLANES;
+            if (Ho > 0 && Wo > 0) variant = FORM_BPLANES;
         }
     }
     if (variant == FORM_BPLANES) return init_batch_planes(state, f, B, H, W, stride, IFMap, OFMap, FORM_BPLANES);
@@ -1001,7 +1003,7 @@ int shflbw_spconv_exec(const shflbw_spconv_state* state, void* stream)
     fill_conv_launch_args(state, &a);
     hipError_t e = hipSuccess;
     if (state->variant == FORM_CHWB || state->variant == FORM_BPLANES) {
-        const ConvChwbKernel* k = conv_chwb_kernel(state->brow);
+        const ConvChwbKernel* k = conv_chwb_kernel(state->brow, state->middle_tile_cols, 0, 0, 0);
         if (!k) return SHFLBW_ERR_UNSUPPORTED;
         const bool nhwc = state->variant == FORM_BPLANES;
         e = nhwc ? launch_nhwc_to_planes(a, (half_t*)state->planes, state->plane_rows, state->plane_cols,

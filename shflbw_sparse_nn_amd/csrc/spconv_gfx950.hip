@@ -782,18 +782,36 @@ static hipError_t prepare_chwb()
             &prepare_chwb<V, WN, NC, NP, KT, NS>                                                                       \
     }
 
+// (the widest tile of a block size first)
 static const ConvChwbKernel g_chwb[] = {
-    SHFLBW_CHWB(64, 128, 4, 4, 32, 4),
-    SHFLBW_CHWB(32, 128, 4, 4, 32, 4),
+    SHFLBW_CHWB(64, 128, 4, 4, 32, 4), SHFLBW_CHWB(64, 64, 4, 4, 32, 6),  SHFLBW_CHWB(64, 32, 4, 4, 32, 6),
+    SHFLBW_CHWB(32, 128, 4, 4, 32, 4), SHFLBW_CHWB(32, 64, 4, 4, 32, 6),  SHFLBW_CHWB(32, 32, 4, 4, 32, 6),
     SHFLBW_CHWB(16, 128, 4, 4, 32, 4),
-    SHFLBW_CHWB(128, 64, 4, 4, 32, 6),
+    SHFLBW_CHWB(128, 64, 4, 4, 32, 6), SHFLBW_CHWB(128, 32, 4, 4, 32, 6),
 };
 
-const ConvChwbKernel* conv_chwb_kernel(int V)
+// The kernel of block height V with tiles of `tile_cols` columns; tile_cols <= 0: the choice for a GEMM of X row panels
+// by `ncols` columns on `cus` compute units, as for the SpMM - 128-column tiles while there are at most as many of them as
+// compute units, 256-column tiles while the 512-column ones would fill at most half of the compute units, the widest
+// otherwise.
+const ConvChwbKernel* conv_chwb_kernel(int V, int tile_cols, long X, long ncols, int cus)
 {
-    for (const ConvChwbKernel& k : g_chwb)
-        if (k.V == V) return &k;
-    return nullptr;
+    const ConvChwbKernel* widest = nullptr;
+    for (const ConvChwbKernel& k : g_chwb) {
+        if (k.V != V) continue;
+        if (!widest) widest = &k;
+        if (k.BN == tile_cols) return &k;
+    }
+    if (tile_cols > 0 || !widest) return nullptr;
+    auto with = [&](int bn) -> const ConvChwbKernel* {
+        for (const ConvChwbKernel& k : g_chwb)
+            if (k.V == V && k.BN == bn) return &k;
+        return nullptr;
+    };
+    const ConvChwbKernel* k = nullptr;
+    if (X * ((ncols + 127) / 128) <= cus && (k = with(128))) return k;
+    if (widest->BN == 512 && X * ((ncols + 511) / 512) <= cus / 2 && (k = with(256))) return k;
+    return widest;
 }
 
 template <int V, int WN, int NCONS, int NPROD, int KT, int NSTAGE>

@@ -94,7 +94,7 @@ struct ConvChwbKernel {
     hipError_t (*launch)(const SpmmLaunchArgs&, hipStream_t);
     hipError_t (*prepare)();
 };
-const ConvChwbKernel* conv_chwb_kernel(int V);
+const ConvChwbKernel* conv_chwb_kernel(int V, int tile_cols, long X, long ncols, int cus);
 
 // Stages 1 and 3 of the plane form of the convolution: NHWC input -> channel-major padded planes (one per
 // stride phase, `copies` = 1 or 2 with a copy moved by one value, rows of `pitch` values), and the

@@ -321,9 +321,9 @@ def test_direct_kernel_names_its_block_sizes(torch_gpu):
     assert e.value.status == capi.ERR_UNSUPPORTED and "32, 64 and 128" in str(e.value)
 
 
-@pytest.mark.parametrize("Bn,H,expected", [(8, 8, 0), (8, 16, 2), (12, 16, 0), (32, 8, 2)])
-def test_the_library_picks_the_batch_innermost_form_for_large_batches_of_eights(torch_gpu, Bn, H, expected):
-    """shflbw_spconv_init: form 2 needs a batch that is a multiple of 8 and pays from 2048 output pixels on."""
+@pytest.mark.parametrize("Bn,H,expected", [(8, 8, 2), (8, 16, 2), (12, 16, 0), (32, 8, 2), (20, 8, 0)])
+def test_the_library_picks_the_batch_innermost_form_for_batches_of_eights(torch_gpu, Bn, H, expected):
+    """shflbw_spconv_init: form 2 needs a batch that is a multiple of 8; other batches get form 0."""
     import shflbw_sparse_nn_amd as S
     torch = torch_gpu
     C, F = 8, 32
@@ -334,3 +334,34 @@ def test_the_library_picks_the_batch_innermost_form_for_large_batches_of_eights(
     op = S.SpconvBlockwiseOp()
     st = op.initialize(f, Bn, H, H, 1, dX.data_ptr(), dY.data_ptr())
     assert st.variant == expected, (Bn * H * H, st.variant)
+
+
+@pytest.mark.parametrize("Bn,H,C,F,V,tile_cols", [
+    (8, 6, 8, 64, 64, 128),       # 1 row panel, 4 tiles of 128 columns
+    (8, 6, 16, 96, 32, 128),
+    (16, 5, 8, 256, 128, 128),
+    (16, 14, 8, 768, 64, 256),    # 12 row panels over 4096 columns: 384 tiles of 128, 96 of 512
+    (16, 14, 8, 384, 32, 256),
+    (16, 14, 8, 640, 32, 512),    # 20 row panels: 160 tiles of 512 columns
+    (16, 14, 8, 1536, 128, 256),  # block height 128 has no wider tile than 256 columns
+    (16, 14, 8, 96, 16, 512),     # block height 16 has the one width
+])
+def test_batch_innermost_form_tile_widths(torch_gpu, Bn, H, C, F, V, tile_cols):
+    """The SpMM in the middle of form 2 takes its tile width from the size of the GEMM (128, 256 or 512 columns, as the
+    SpMM proper does); every width gives the oracle's bits."""
+    import shflbw_sparse_nn_amd as S
+    torch = torch_gpu
+    w = P.make_weight(F, 9 * C, V, 0.4, True, 77, integer=True)
+    x = np.random.default_rng(78).integers(-4, 5, size=(Bn, H, H, C)).astype(np.float16)
+    ref = O.float_to_half(P.conv_oracle(w, 3, 3, C, x, 1))
+    f = P.upload_weight(w, 3, 3, C, cls=S.BlockwiseSpFilter)
+    dX = P.to_dev(torch, x)
+    dY = torch.full((Bn, H, H, F), float("nan"), dtype=torch.float16, device="cuda")
+    op = S.SpconvBlockwiseOp(2)
+    st = op.initialize(f, Bn, H, H, 1, dX.data_ptr(), dY.data_ptr())
+    assert st.middle_tile_cols == tile_cols
+    print("conv form 2", (Bn, H, C, F, V), "tiles of", st.middle_tile_cols, "columns, grid", st.grid_dim[0], flush=True)
+    op(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    op.check()
+    np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16))
