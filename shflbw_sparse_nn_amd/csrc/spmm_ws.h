@@ -4,6 +4,9 @@
 // fragments).  Replaces, together with the kernels built from it, the reference's main loop and device
 // primitives (block_sparse/spmm/blockwise_kernel.h:108-294, block_sparse/common/{mma,memcpy,swizzle,epilogue}.h).
 #pragma once
+#ifndef SHFLBW_EPI_LINES
+#define SHFLBW_EPI_LINES 1
+#endif
 #include <type_traits>
 
 #include "kernel_common.h"
@@ -283,8 +286,73 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
         const uint32_t rd = epi + (lane / PR) * Cfg::EPI_ROWB + pc * 16;
         // specialised on "alpha == 1" and "beta == 0" so that the common path has no branch (a
         // branch per piece would put a full wait at every join)
+        // Whole lines: with an even number of 32-column blocks, 16 rows of two neighbouring blocks are staged at a time
+        // (rows of 128 bytes + 16) and eight lanes store one 128-byte line of a row: half as many write requests to the
+        // L2s as with 64-byte row segments (cfg1 -2 %, 11 % at N = 16384, where every epilogue runs beside other
+        // workgroups' gathers).  Not where two workgroups share a compute unit (128 registers per wave: it spills).
+        constexpr bool LINES = SHFLBW_EPI_LINES && NB % 2 == 0 && 16 * (128 + 16) <= Cfg::EPI_WAVE_BYTES && Cfg::WGS_PER_CU == 1;
+        constexpr int LROWB = 128 + 16;
+        const uint32_t wrl = epi + (lane & 15) * LROWB + (lane >> 5) * 8;
+        const uint32_t rdl = epi + (lane >> 3) * LROWB + (lane & 7) * 16;
+        auto epi_lines = [&](int mb, auto scale, auto add_c) __attribute__((always_inline)) {
+            constexpr bool SCALE = decltype(scale)::value, ADDC = decltype(add_c)::value;
+#pragma unroll
+            for (int np = 0; np < NB / 2; np++)
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) { // rows 16 hh .. 16 hh + 15 of the block: the lanes with bit 4 equal to hh
+                    size_t roff[2];
+#pragma unroll
+                    for (int it = 0; it < 2; it++) {
+                        const int rr = mb * 32 + hh * 16 + it * 8 + (lane >> 3);
+                        roff[it] = (size_t)__shfl(rid[rr >> 6], rr & 63) * a.ldd;
+                    }
+                    if (((lane >> 4) & 1) == hh) {
+#pragma unroll
+                        for (int nb2 = 0; nb2 < 2; nb2++)
+#pragma unroll
+                            for (int ig = 0; ig < 4; ig++) {
+                                half4_t h;
+#pragma unroll
+                                for (int e = 0; e < 4; e++) {
+                                    const float x = acc[mb][np * 2 + nb2][ig * 4 + e];
+                                    h[e] = (half_t)(SCALE ? x * alpha : x);
+                                }
+                                *(SHFLBW_LDS half4_t*)(uintptr_t)(wrl + nb2 * 64 + ig * 16) = h;
+                            }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    half8_t v[2], c[2];
+#pragma unroll
+                    for (int it = 0; it < 2; it++) v[it] = *(SHFLBW_LDS half8_t*)(uintptr_t)(rdl + it * 8 * LROWB);
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier(); // the next 16 rows overwrite what other lanes have just read
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    int col = n0 + cw * WN + np * 64 + (lane & 7) * 8;
+                    bool keep = col < N;
+                    if (DMAP) keep = keep && output_column(a, col);
+                    if (keep) {
+                        if (ADDC) {
+#pragma unroll
+                            for (int it = 0; it < 2; it++) c[it] = *(const half8_t*)(a.C + roff[it] + col);
+#pragma unroll
+                            for (int it = 0; it < 2; it++)
+#pragma unroll
+                                for (int e = 0; e < 8; e++)
+                                    v[it][e] = (half_t)((float)v[it][e] + beta * (float)c[it][e]);
+                        }
+#pragma unroll
+                        for (int it = 0; it < 2; it++) store_result_16B<!XCD_LOCAL>(a.D + roff[it] + col, v[it]);
+                    }
+                }
+        };
         auto epi_block = [&](int mb, auto scale, auto add_c) __attribute__((always_inline)) {
             constexpr bool SCALE = decltype(scale)::value, ADDC = decltype(add_c)::value;
+            if constexpr (LINES) {
+                epi_lines(mb, scale, add_c);
+                return;
+            }
 #pragma unroll
             for (int hh = 0; hh < 32 / ER; hh++) {
                 size_t roff[NIT]; // element offset of the lane's output row, without the column
