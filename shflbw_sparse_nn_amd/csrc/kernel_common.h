@@ -101,6 +101,14 @@ __device__ __forceinline__ void store_result_16B(half_t* p, half8_t v)
         asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
+// alpha * acc as the reference's `d * alpha + c * beta` leaves it (spmm/blockwise_format.h:307): without a C term the sum
+// is `d * alpha + (+0)`, which turns a product of -0 (a zero accumulator under a negative alpha) into +0; with a C term
+// the product goes on unchanged (x + (-0) == x for every x).  One fused multiply-add either way.
+__device__ __forceinline__ float scaled(float acc, float alpha, bool c_term_follows)
+{
+    return __builtin_fmaf(acc, alpha, c_term_follows ? -0.f : 0.f);
+}
+
 // Words that workgroups of one launch count in (queues, arrival counts) are kept one cache line apart: atomics on
 // one line are served one after the other (about 11 ns each with every compute unit taking part).
 constexpr int SYNC_LINE = 64; // ints

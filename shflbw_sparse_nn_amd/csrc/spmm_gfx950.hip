@@ -211,7 +211,7 @@ __global__ void __launch_bounds__(NWAVES * 64) spmm_shflbw_kernel(SpmmLaunchArgs
             for (int ig = 0; ig < 4; ig++) {
                 half4_t h;
 #pragma unroll
-                for (int e = 0; e < 4; e++) h[e] = (half_t)(acc[mb][nb][ig * 4 + e] * alpha);
+                for (int e = 0; e < 4; e++) h[e] = (half_t)scaled(acc[mb][nb][ig * 4 + e], alpha, a.beta != 0.f);
                 const int m = mb * 32 + (lane & 31);
                 const int n = wave * WN + nb * 32 + ig * 8 + (lane >> 5) * 4;
                 *(SHFLBW_LDS half4_t*)(uintptr_t)(lds0 + m * EPI_ROWB + n * 2) = h;

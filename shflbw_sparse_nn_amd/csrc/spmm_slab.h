@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(SpmmSlabCfg::THREADS) spmm_shflbw_slab_kernel(
                         for (int ig = 0; ig < 4; ig++) {
                             half4_t h;
 #pragma unroll
-                            for (int e = 0; e < 4; e++) h[e] = (half_t)(acc[nb][ig * 4 + e] * alpha);
+                            for (int e = 0; e < 4; e++) h[e] = (half_t)scaled(acc[nb][ig * 4 + e], alpha, beta != 0.f);
                             *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + nb * 64 + ig * 16) = h;
                         }
                 }

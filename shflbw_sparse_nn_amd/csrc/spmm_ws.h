@@ -315,7 +315,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
 #pragma unroll
                                 for (int e = 0; e < 4; e++) {
                                     const float x = acc[mb][np * 2 + nb2][ig * 4 + e];
-                                    h[e] = (half_t)(SCALE ? x * alpha : x);
+                                    h[e] = (half_t)(SCALE ? scaled(x, alpha, ADDC) : x);
                                 }
                                 *(SHFLBW_LDS half4_t*)(uintptr_t)(wrl + nb2 * 64 + ig * 16) = h;
                             }
@@ -369,7 +369,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmLaunchArgs& a, uint32_t ld
                             half4_t h;
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                h[e] = (half_t)(SCALE ? acc[mb][nb][ig * 4 + e] * alpha : acc[mb][nb][ig * 4 + e]);
+                                h[e] = (half_t)(SCALE ? scaled(acc[mb][nb][ig * 4 + e], alpha, ADDC) : acc[mb][nb][ig * 4 + e]);
                             *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + ig * 16) = h;
                         }
                     }
@@ -520,7 +520,7 @@ __device__ __forceinline__ void ws_consumer16(const SpmmLaunchArgs& a, uint32_t 
             for (int q = 0; q < 4; q++) {
                 half4_t hv;
 #pragma unroll
-                for (int e = 0; e < 4; e++) hv[e] = (half_t)(acc[h * 4 + q][e] * alpha);
+                for (int e = 0; e < 4; e++) hv[e] = (half_t)scaled(acc[h * 4 + q][e], alpha, beta != 0.f);
                 *(SHFLBW_LDS half4_t*)(uintptr_t)(wr + q * 32) = hv;
             }
             half8_t v[2];

@@ -365,3 +365,38 @@ def test_batch_innermost_form_tile_widths(torch_gpu, Bn, H, C, F, V, tile_cols):
     torch.cuda.synchronize()
     op.check()
     np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_library_choice_seeded_random_shapes(torch_gpu):
+    """Twenty-four seeded NHWC problems with the form the library picks (form 2 for batches of eights, form 0 otherwise;
+    the SpMM in the middle with tiles of 128, 256 or 512 columns): filter extents 1..5, strides 1..3, all block heights."""
+    import shflbw_sparse_nn_amd as S
+    torch = torch_gpu
+    rng = np.random.default_rng(2718)
+    forms = set()
+    for case in range(24):
+        V = int(rng.choice([16, 32, 64, 128]))
+        F = V * int(rng.integers(1, 6))
+        C = 8 * int(rng.integers(1, 6))  # the NHWC forms move channels in eights
+        R, S_ = int(rng.choice([1, 3, 5])), int(rng.choice([1, 2, 3, 5]))
+        H, W = int(rng.integers(3, 20)), int(rng.integers(3, 20))
+        Bn = int(rng.choice([1, 2, 3, 8, 16, 24, 40]))
+        stride = int(rng.integers(1, 4))
+        d = float(rng.choice([0.1, 0.4, 1.0]))
+        w = P.make_weight(F, R * S_ * C, V, d, bool(rng.integers(0, 2)), 900 + case, integer=True)
+        x = rng.integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
+        ref = O.float_to_half(P.conv_oracle(w, R, S_, C, x, stride))
+        f = P.upload_weight(w, R, S_, C, cls=S.BlockwiseSpFilter)
+        dX = P.to_dev(torch, x)
+        dY = torch.full(ref.shape, float("nan"), dtype=torch.float16, device="cuda")
+        op = S.SpconvBlockwiseOp()
+        st = op.initialize(f, Bn, H, W, stride, dX.data_ptr(), dY.data_ptr())
+        forms.add(st.variant)
+        print("case", case, (Bn, H, W, C, F, R, S_, stride, V, d), "form", st.variant, "tiles of", st.middle_tile_cols, flush=True)
+        assert op.output_hw == ref.shape[1:3]
+        op(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        op.check()
+        np.testing.assert_array_equal(dY.cpu().numpy().view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
+    assert forms == {0, 2}
+

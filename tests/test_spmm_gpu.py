@@ -267,3 +267,40 @@ def test_slab_variant_seeded_random_shapes(torch_gpu):
         got = run_spmm(torch_gpu, w, B, Cmat=Cm, variant=v)
         ref = O.float_to_half(P.spmm_oracle(w, B, Cm, 1.0, 1.0) if with_c else P.spmm_oracle(w, B))
         np.testing.assert_array_equal(got.view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
+
+
+def test_library_choice_seeded_random_shapes(torch_gpu):
+    """Forty seeded shapes over every block height with the variant the library picks (tiles of 128, 256 or 512 columns
+    by the size of the problem, the slab kernel where it applies): ragged N, K not a multiple of anything, densities
+    from nearly empty to full, permuted or not, with and without C and a scale: bit-exact against the oracle."""
+    import shflbw_sparse_nn_amd as S
+    rng = np.random.default_rng(31415)
+    seen = set()
+    for case in range(40):
+        V = int(rng.choice([16, 32, 64, 128]))
+        M = V * int(rng.integers(1, 24))
+        K = int(rng.integers(1, 700))
+        N = 8 * int(rng.integers(1, 400))
+        d = float(rng.choice([0.02, 0.1, 0.3, 0.6, 1.0]))
+        permute = bool(rng.integers(0, 2))
+        with_c = bool(rng.integers(0, 2))
+        alpha = float(rng.choice([1.0, 2.0, -0.5]))
+        w = P.make_weight(M, K, V, d, permute, 500 + case, integer=True)
+        B = P.make_dense(K, N, 500 + case, integer=True)
+        Cm = P.make_dense(M, N, 500 + case, integer=True, stream=3) if with_c else None
+        m = P.upload_weight(w)
+        dB = P.to_dev(torch_gpu, B)
+        dC = None if Cm is None else P.to_dev(torch_gpu, Cm)
+        dD = torch_gpu.full((M, N), float("nan"), dtype=torch_gpu.float16, device="cuda")
+        op = S.SpmmBlockwiseOp()
+        st = op.initialize(m, N, dB.data_ptr(), dD.data_ptr(), None if dC is None else dC.data_ptr(), alpha, 1.0 if with_c else 0.0)
+        name = S.spmm_variants(V)[st.variant]
+        seen.add(name)
+        print("case", case, (M, N, K, V, d, permute, with_c, alpha), name, flush=True)
+        op(torch_gpu.cuda.current_stream().cuda_stream)
+        torch_gpu.cuda.synchronize()
+        ref = O.float_to_half(P.spmm_oracle(w, B, Cm, alpha, 1.0) if with_c else P.spmm_oracle(w, B, None, alpha, 0.0))
+        np.testing.assert_array_equal(dD.cpu().numpy().view(np.uint16), ref.view(np.uint16), err_msg="case %d" % case)
+    print("variants met:", sorted(seen), flush=True)
+    assert len(seen) >= 6
+
