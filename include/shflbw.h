@@ -208,7 +208,7 @@ const char* shflbw_spmm_variant_name(int brow, int variant);
  *     planes (one per stride phase); the SpMM kernel then gathers, for a kept k = (r, s, c), the
  *     plane of channel c at the constant offset of tap (r, s) - the im2col matrix is never built,
  *     its address generation is the per-id offset of the gather; a tile transpose writes NHWC;
- *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads; block sizes 32, 64, 128);
+ *   variant 1 = a single direct kernel (im2col gather from NHWC in the tile loads; every block size);
  *   variant 2 = plane form with the batch innermost in the planes and in the filter-major result (B % 8 == 0):
  *     every tap offset is then a multiple of 16 bytes, one copy of the planes serves all taps, and the result
  *     holds output pixels only; three launches;

@@ -473,7 +473,7 @@ int spconv_fill_state(shflbw_spconv_state* state, const shflbw_weight* f, int B,
     if (variant == FORM_DIRECT) {
         const SpconvVariant* v = find_spconv_variant(f->brow, 0, nullptr);
         if (!v) {
-            set_error("spconv_init: the direct kernel (variant 1) exists for block sizes 32, 64 and 128, not %d; "
+            set_error("spconv_init: the direct kernel (variant 1) exists for block sizes 16, 32, 64 and 128, not %d; "
                       "the plane forms (0, 2, 3) serve every block size", f->brow);
             return SHFLBW_ERR_UNSUPPORTED;
         }

@@ -18,8 +18,9 @@ namespace shflbw {
 template <int V, int WN, int NWAVES, int KT>
 struct SpconvCfg {
     static constexpr int BN = WN * NWAVES;
-    static constexpr int MB = V / 32;
+    static constexpr int MB = V / 32;   // 32-row blocks of a panel (block height 16: none, one 16x16x32 tile row)
     static constexpr int NB = WN / 32;
+    static constexpr int NB16 = WN / 16; // 16-column blocks of a wave (block height 16)
     static constexpr int ROWB = BN * 2;
     static constexpr int CPR = BN / 8;
     static constexpr int SPT = KT / 16;
@@ -28,7 +29,7 @@ struct SpconvCfg {
     static constexpr int PPT = PIECES / THREADS;     // pieces per thread
     static constexpr int ROWS_PER_PASS = THREADS / CPR;
     static constexpr int LDS_BYTES = KT * ROWB;
-    static_assert(V % 32 == 0 && WN % 32 == 0, "32x32x16 tiles");
+    static_assert((V % 32 == 0 || (V == 16 && KT == 32)) && WN % 32 == 0, "32x32x16 tiles, or 16x16x32 for V = 16");
     static_assert(BN >= 128 && BN <= 512 && (BN & (BN - 1)) == 0, "row swizzle range");
     static_assert(PIECES % THREADS == 0 && THREADS % CPR == 0 && ROWS_PER_PASS % 4 == 0,
                   "a thread keeps one column piece and a fixed row phase across passes");
@@ -40,6 +41,8 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
     using Cfg = SpconvCfg<V, WN, NWAVES, KT>;
     constexpr int BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, ROWB = Cfg::ROWB, CPR = Cfg::CPR, SPT = Cfg::SPT;
     constexpr int PPT = Cfg::PPT, RPP = Cfg::ROWS_PER_PASS;
+    constexpr bool V16 = V == 16;       // 16x16x32 tiles: one 32-slot step per A fragment, a lane holds 4 pixels of one filter
+    constexpr int NB16 = Cfg::NB16;
 
     extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(SHFLBW_LDS char*)lds_raw;
@@ -89,13 +92,23 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
         boff[nb] = (uint32_t)((8 * (lane >> 5) + (li >> 2)) * ROWB + ((unit ^ row_xor32(li >> 2)) << 5) + ((li & 3) << 3));
     }
 
-    float16_t acc[MB][NB];
+    float16_t acc[V16 ? 1 : MB][NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int mb = 0; mb < (V16 ? 1 : MB); mb++)
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mb][nb][i] = 0.f;
+    // block height 16: the fragment addresses and accumulators of the 16x16x32 tiles (as in the SpMM's consumer for
+    // that block height: rows 8 (lane / 16) + (lane % 16) / 4 and four further down, 16-column units)
+    uint32_t boff16[NB16];
+    float4_t acc16[NB16];
+#pragma unroll
+    for (int nb = 0; nb < NB16; nb++) {
+        const int unit = (wave * WN + nb * 16) / 16;
+        boff16[nb] = (uint32_t)((8 * (lane >> 4) + (li >> 2)) * ROWB + ((unit ^ row_xor32(li >> 2)) << 5) + ((li & 3) << 3));
+        acc16[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     const int SC = a.S * a.C;
     for (int t = 0; t < ntiles; t++) {
@@ -119,6 +132,19 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
             *(SHFLBW_LDS half8_t*)(uintptr_t)(lds0 + wr_off + j * RPP * ROWB) = piece[j];
         __syncthreads();
 
+        if constexpr (V16) { // one 32-slot step per stage; an odd last 16-slot step has zero weights behind it
+            static_assert(!V16 || SPT == 2, "a stage is one 32-slot step");
+            if (t * SPT < nsteps) {
+                const half8_t afrag = pA[(size_t)t * 64 + lane];
+#pragma unroll
+                for (int nb = 0; nb < NB16; nb++) {
+                    const half4_t lo = lds_read_tr16(lds0 + boff16[nb]);
+                    const half4_t hi = lds_read_tr16(lds0 + boff16[nb] + 4 * ROWB);
+                    const half8_t bfrag = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc16[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bfrag, afrag, acc16[nb], 0, 0, 0);
+                }
+            }
+        } else
 #pragma unroll
         for (int kk = 0; kk < SPT; kk++) {
             const int step = t * SPT + kk;
@@ -142,7 +168,19 @@ __global__ void __launch_bounds__(NWAVES * 64) spconv_shflbw_kernel(SpconvLaunch
     }
 
     // ---- epilogue: one fp32 -> fp16 rounding, NHWC store; a lane holds output channel
-    // perm[panel*V + mb*32 + lane%32] of 16 pixels per 32x32 block
+    // perm[panel*V + mb*32 + lane%32] of 16 pixels per 32x32 block (block height 16: channel perm[panel*16 + lane%16]
+    // of 4 pixels per 16x16 block)
+    if constexpr (V16) {
+        const int srow = panel * V + (lane & 15);
+        const int f = a.row_ids ? a.row_ids[srow] : srow;
+#pragma unroll
+        for (int nb = 0; nb < NB16; nb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int p = n0 + wave * WN + nb * 16 + (lane >> 4) * 4 + i;
+                if (p < npix) a.out[(size_t)p * a.F + f] = (half_t)acc16[nb][i];
+            }
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
         const int srow = panel * V + mb * 32 + (lane & 31);
@@ -893,6 +931,7 @@ static const SpconvVariant g_conv_variants[] = {
     SHFLBW_CONV_VARIANT(64, 32, 4, 32),
     SHFLBW_CONV_VARIANT(32, 32, 4, 32),
     SHFLBW_CONV_VARIANT(128, 32, 4, 32),
+    SHFLBW_CONV_VARIANT(16, 32, 4, 32),
 };
 
 const SpconvVariant* spconv_variants(int* count)

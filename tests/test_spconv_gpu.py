@@ -19,9 +19,9 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     w = P.make_weight(F, R * S * C, V, d, permute, seed, integer=True)
     x = np.random.default_rng(seed + 1).integers(-4, 5, size=(Bn, H, W, C)).astype(np.float16)
     ref = O.float_to_half(P.conv_oracle(w, R, S, C, x, stride))
-    # 0: plane layout + SpMM + transpose, 1: one direct kernel (block heights 32, 64, 128); batches that are multiples of 8
+    # 0: plane layout + SpMM + transpose, 1: one direct kernel; batches that are multiples of 8
     # also 2: planes and result with the batch innermost, 3: the steps of 2 in one launch, every XCD on its own columns
-    forms = (0, 1) if V != 16 else (0,)
+    forms = (0, 1)
     if Bn % 8 == 0:
         forms += (2, 3)
     for variant in forms:
@@ -38,7 +38,7 @@ def _exact(torch, Bn, H, W, C, F, R, S, stride, V, d, permute=True, seed=2021):
     (3, 9, 9, 8, 128, 1, 1, 1, 128, 0.6, False),  # 1x1 filter, no permutation
     (2, 8, 8, 24, 64, 5, 3, 1, 32, 0.2, True),    # rectangular filter
     (4, 14, 14, 64, 128, 3, 3, 2, 64, 0.05, True),
-    (2, 9, 7, 16, 48, 3, 3, 1, 16, 0.4, True),    # block height 16 (no direct kernel)
+    (2, 9, 7, 16, 48, 3, 3, 1, 16, 0.4, True),    # block height 16
     (2, 12, 10, 8, 64, 5, 5, 2, 32, 0.3, True),   # 5x5 stride 2: tap offsets 0..2 inside a phase plane
     (1, 11, 9, 16, 64, 3, 3, 3, 64, 0.5, True),   # stride 3: nine phase planes, one tap each
     (2, 6, 20, 8, 32, 1, 7, 1, 32, 0.4, True),    # 1x7 filter: seven tap offsets in one row
@@ -312,13 +312,17 @@ def test_batch_innermost_forms_need_a_batch_of_eights(torch_gpu, variant):
     assert e.value.status == capi.ERR_SHAPE
 
 
-def test_direct_kernel_names_its_block_sizes(torch_gpu):
+def test_direct_kernel_refuses_inputs_it_cannot_index(torch_gpu):
+    """The direct kernel (every block height has one) indexes the input with 32 bits and says so in init."""
+    import shflbw_sparse_nn_amd as S
     from shflbw_sparse_nn_amd import capi
     w = P.make_weight(64, 9 * 8, 16, 0.3, True, 3, integer=True)
-    x = np.zeros((2, 5, 5, 8), dtype=np.float16)
+    f = P.upload_weight(w, 3, 3, 8, cls=S.BlockwiseSpFilter)
+    op = S.SpconvBlockwiseOp(1)
+    t = torch_gpu.zeros(8, dtype=torch_gpu.float16, device="cuda")
     with pytest.raises(capi.ShflbwError) as e:
-        run_spconv(torch_gpu, w, 3, 3, 8, x, 1, 1)
-    assert e.value.status == capi.ERR_UNSUPPORTED and "32, 64 and 128" in str(e.value)
+        op.initialize(f, 1 << 12, 1 << 8, 1 << 8, 1, t.data_ptr(), t.data_ptr())  # 2^31 input values; init reads no tensor
+    assert e.value.status == capi.ERR_UNSUPPORTED and "2^31" in str(e.value)
 
 
 @pytest.mark.parametrize("Bn,H,expected", [(8, 8, 2), (8, 16, 2), (12, 16, 0), (32, 8, 2), (20, 8, 0)])
